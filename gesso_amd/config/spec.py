@@ -31,6 +31,17 @@ class RMSNormSpec:
 
 
 @dataclass(frozen=True)
+class GroupRMSNormSpec:
+    """RMS norm in parts: the row is cut into ``groups`` equal consecutive parts, each is divided by its own
+    ``sqrt(mean(part^2) + eps)``, and the whole is multiplied by the weight."""
+
+    size: int
+    eps: float
+    groups: int = 1
+    kind: str = "group_rmsnorm"
+
+
+@dataclass(frozen=True)
 class RopeSpec:
     """Rotary encoding over the first ``rotary_dim`` features of a head; ``layout``: pairs ``(i, i + rotary_dim/2)``
     (``"half"``) or ``(2i, 2i + 1)`` (``"interleaved"``)."""
@@ -118,7 +129,9 @@ class LatentAttentionSpec:
     of all heads from one normed latent row of ``kv_rank`` features per token, plus ``rot_dim`` rotated key features
     that all heads share.  A head has ``plain_dim`` unrotated and ``rot_dim`` rotated query/key features (in that
     order) and ``value_dim`` value features.  ``gated``: head ``h``'s output is multiplied by
-    ``sigmoid(W_g x)[h]``.  ``position`` is the encoding of the ``rot_dim`` part (its ``head_dim`` = ``rot_dim``)."""
+    ``sigmoid(W_g x)[h]``; with ``gate_each`` every output feature has a gate of its own (``W_g`` has
+    ``n_heads * value_dim`` rows).  ``position`` is the encoding of the ``rot_dim`` part (its ``head_dim`` = ``rot_dim``);
+    its pairs may be laid out either way."""
 
     hidden: int
     n_heads: int
@@ -133,6 +146,7 @@ class LatentAttentionSpec:
     window: Optional[int] = None       # keys a query sees, itself included; None = all
     gated: bool = True
     kind: str = "latent_attention"
+    gate_each: bool = False
 
 
 @dataclass(frozen=True)
@@ -218,6 +232,49 @@ class TableMoESpec:
 
 
 @dataclass(frozen=True)
+class StateSpaceSpec:
+    """A state-space mixer whose decay and step size depend on the token.  ``inner = n_heads * head_dim``; the input
+    product gives ``[z: inner | x: inner | B: groups * state | C: groups * state | dt: n_heads]``; x, B and C pass a causal
+    convolution of ``conv_taps`` taps per channel (with a bias) and silu; ``dt = softplus(dt + dt_bias)``; per head ``h``
+    (group ``h // (n_heads / groups)``) ``S_t = exp(-exp(A_log[h]) dt_t) S_(t-1) + dt_t B_t x_t^T`` (``state x head_dim``,
+    float32, zero at a request's start), ``y_t = S_t^T C_t + D[h] x_t``; ``y * silu(z)`` is RMS-normed in ``norm_groups``
+    equal parts, times a weight, and projected back."""
+
+    hidden: int
+    n_heads: int
+    head_dim: int
+    state: int
+    groups: int
+    norm_groups: int
+    conv_taps: int
+    eps: float
+    kind: str = "state_space"
+
+
+@dataclass(frozen=True)
+class RoutedMoESpec:
+    """A mixture of gated feed-forwards chosen by a router over the token's features.  The router has
+    ``n_experts + n_identity`` outputs; its scores are their softmax; the ``top`` outputs with the largest
+    score + ``correction`` (a stored vector, when ``correction``) are chosen and weighted by their scores divided by the
+    chosen scores' sum (+ 1e-20).  The last ``n_identity`` outputs name no weights: such an expert gives back its input.
+    An expert is ``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate x, limit)``,
+    ``u = clamp(W_up x, -limit, limit)``.  ``shared_ff``: a further expert of that width and ``shared_limit`` runs for every
+    token and is added (None: none)."""
+
+    hidden: int
+    n_experts: int
+    top: int
+    expert_ff: int
+    limit: float
+    n_identity: int = 0
+    alpha: float = 1.702
+    correction: bool = True
+    shared_ff: Optional[int] = None
+    shared_limit: Optional[float] = None
+    kind: str = "routed_moe"
+
+
+@dataclass(frozen=True)
 class BlockSpec:
     """One block: ``h += mixer(norm(h)); h += ffn(norm(h))`` for ``arrangement="prenorm"``.
 
@@ -262,6 +319,31 @@ class ParallelBlockSpec:
 
 
 @dataclass(frozen=True)
+class SharedNormBlockSpec:
+    """One block with a single norm that both sub-layers read: with ``a = norm(h)``,
+    ``h += mixer(a + conv(a)) + ffn(a)``.  ``input_taps``: the mixer's input gets a causal convolution over time added
+    to it, ``conv(a)_t = sum_j w[:, j] a_(t - taps + 1 + j)`` per channel, no bias (None: the mixer reads ``a`` itself); its
+    last ``taps - 1`` inputs are part of a request's state.  ``names`` as in :class:`BlockSpec` (roles ``norm.``,
+    ``input_conv.``, ``mixer.``, ``ffn.``)."""
+
+    mixer: Any
+    norm: Any
+    ffn: Any                           # None = no feed-forward in this block
+    input_taps: Optional[int] = None
+    names: Mapping[str, str] = field(compare=False, hash=False, default_factory=dict)
+    kind: str = "shared_norm"
+
+
+@dataclass(frozen=True)
+class ReentrySpec:
+    """Before the schedule entries ``at`` (in their order, ``t = 0, 1, ...``) the stream is mixed with the embedding
+    output ``x0`` again: ``x <- W [x; x0] + step[t]`` with ``W (hidden, 2 hidden)`` (the stream's columns first) and
+    ``step (len(at), hidden)``.  The model's names ``reentry.weight`` and ``reentry.step`` say where they are stored."""
+
+    at: Tuple[int, ...]
+
+
+@dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order: block ``layer`` runs here.
 
@@ -291,6 +373,7 @@ class ModelSpec:
     embed_norm: Any = None                  # a norm spec: the embedding rows are normed before the first block
                                             # (its tensors under names "embed_norm.<local>")
     logit_softcap: Optional[float] = None   # logits = cap * tanh(logits / cap) (None: as they are)
+    reentry: Optional[ReentrySpec] = None   # see :class:`ReentrySpec`
 
     def __post_init__(self):
         n = len(self.blocks)
@@ -299,3 +382,7 @@ class ModelSpec:
                 raise ValueError(f"schedule entry {i} names block {call.layer}, there are {n}")
             if call.cache is not None and not 0 <= call.cache < i:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {call.cache}, which does not run before it")
+        if self.reentry is not None:
+            at = tuple(self.reentry.at)
+            if not at or list(at) != sorted(set(at)) or not 0 <= at[0] <= at[-1] < len(self.schedule):
+                raise ValueError(f"re-entry points {at} must be distinct schedule entries in ascending order")

@@ -10,7 +10,8 @@
 //                     key/value latent, rotation of the shared key features, both into the token's cache row
 //   latent_q_rot      rotates the rotated part of every head's query into its place behind the absorbed part
 //   heads_product     Y[t, h, :] = W[h] X[t, h, :] for all heads in one launch, with an optional gate: times
-//                     sigmoid(G[t, h]); float32 FMAs in a fixed summation order, or the matrix cores for bfloat16
+//                     sigmoid(G[t, h]), or times sigmoid(G[t, h N + n]) for output n (a gate each); float32 FMAs in a
+//                     fixed summation order, or the matrix cores for bfloat16
 //   attention_latent  the general attention kernel over such rows: any sizes, float32 arithmetic
 //
 // All norms, angles, scores, softmax weights and the gate's sigmoid are float32.
@@ -124,8 +125,8 @@ extern "C" int gs_latent_q_rot(const void* q, int dtype, int ldq, int H, int n, 
 
 template <typename TX, typename TW>
 __global__ void heads_product_kernel(const TX* __restrict__ X, int ldx, int hx, const TW* __restrict__ W,
-                                     TX* __restrict__ Y, int ldy, int hy, const TX* __restrict__ G, int ldg, int M,
-                                     int N, int K) {
+                                     TX* __restrict__ Y, int ldy, int hy, const TX* __restrict__ G, int ldg,
+                                     int gate_each, int M, int N, int K) {
   __shared__ float xs[HP_TK][HP_TM + 4];
   __shared__ float ws[HP_TK][HP_TN + 4];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
@@ -175,11 +176,13 @@ __global__ void heads_product_kernel(const TX* __restrict__ X, int ldx, int hx, 
     const int m = m0 + ty * 4 + i;
     if (m >= M) continue;
     float gate = 1.f;
-    if (G) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
+    if (G && !gate_each) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) Y[(size_t)m * ldy + n] = from_f32<TX>(tot[i][j] * gate);
+      if (n >= N) continue;
+      if (G && gate_each) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + (size_t)h * N + n])));
+      Y[(size_t)m * ldy + n] = from_f32<TX>(tot[i][j] * gate);
     }
   }
 }
@@ -196,7 +199,7 @@ template <int NTW, int MTW>
 __global__ __launch_bounds__(256) void heads_product_mfma_kernel(const bf16* __restrict__ X, int ldx, int hx,
                                                                  const bf16* __restrict__ W, bf16* __restrict__ Y,
                                                                  int ldy, int hy, const bf16* __restrict__ G, int ldg,
-                                                                 int M, int N, int K) {
+                                                                 int gate_each, int M, int N, int K) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
   const int mtiles = (M + 16 * MTW - 1) / (16 * MTW), ngroups = (N + 16 * NTW - 1) / (16 * NTW);
@@ -250,23 +253,25 @@ __global__ __launch_bounds__(256) void heads_product_mfma_kernel(const bf16* __r
       const int m = m0 + 16 * i + 4 * g + e;
       if (m >= M) continue;
       float gate = 1.f;
-      if (G) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
+      if (G && !gate_each) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + h])));
 #pragma unroll
       for (int j = 0; j < NTW; ++j) {
         const int n = n0 + 16 * j + r16;
-        if (n < N) Y[(size_t)m * ldy + (size_t)h * hy + n] = f32_to_bf16(acc[i][j][e] * gate);
+        if (n >= N) continue;
+        if (G && gate_each) gate = 1.f / (1.f + expf(-to_f32(G[(size_t)m * ldg + (size_t)h * N + n])));
+        Y[(size_t)m * ldy + (size_t)h * hy + n] = f32_to_bf16(acc[i][j][e] * gate);
       }
     }
 }
 
 extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, const void* W, int w_dtype, void* Y,
-                                int ldy, int hy, const void* G, int ldg, int M, int N, int K, int H,
+                                int ldy, int hy, const void* G, int ldg, int gate_each, int M, int N, int K, int H,
                                 hipStream_t stream) {
   GS_REQUIRE(M >= 0 && N > 0 && K > 0 && H > 0, "heads_product: bad sizes M=%d N=%d K=%d H=%d", M, N, K, H);
   GS_REQUIRE(H <= 65535 && gs_ceil_div(M, HP_TM) <= 65535, "heads_product: too many heads or rows for one launch");
   GS_REQUIRE((long)(H - 1) * hx + K <= ldx && (long)(H - 1) * hy + N <= ldy,
              "heads_product: heads reach past their rows (ldx=%d hx=%d K=%d, ldy=%d hy=%d N=%d)", ldx, hx, K, ldy, hy, N);
-  GS_REQUIRE(G == nullptr || ldg >= H, "heads_product: gate rows of %d hold no %d heads", ldg, H);
+  GS_REQUIRE(G == nullptr || ldg >= (gate_each ? H * N : H), "heads_product: gate rows of %d hold no gates for %d heads", ldg, H);
   if (M == 0) return 0;
   if (x_dtype == GS_BF16 && w_dtype == GS_BF16 && K % 8 == 0 && ldx % 8 == 0 && hx % 8 == 0 && ((uintptr_t)X & 15) == 0 &&
       ((uintptr_t)W & 15) == 0) {
@@ -278,23 +283,23 @@ extern "C" int gs_heads_product(const void* X, int x_dtype, int ldx, int hx, con
     dim3 grid((unsigned)gs_ceil_div(items, 4), H);
     if (ntw == 1)
       heads_product_mfma_kernel<1, 1><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
-                                                            (const bf16*)G, ldg, M, N, K);
+                                                            (const bf16*)G, ldg, gate_each, M, N, K);
     else
       heads_product_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy, hy,
-                                                            (const bf16*)G, ldg, M, N, K);
+                                                            (const bf16*)G, ldg, gate_each, M, N, K);
     GS_LAUNCH_CHECK("heads_product_mfma");
     return 0;
   }
   dim3 grid(gs_ceil_div(N, HP_TN), gs_ceil_div(M, HP_TM), H);
   if (x_dtype == GS_F32 && w_dtype == GS_F32)
     heads_product_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)X, ldx, hx, (const float*)W, (float*)Y,
-                                                                 ldy, hy, (const float*)G, ldg, M, N, K);
+                                                                 ldy, hy, (const float*)G, ldg, gate_each, M, N, K);
   else if (x_dtype == GS_BF16 && w_dtype == GS_BF16)
     heads_product_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const bf16*)W, (bf16*)Y, ldy,
-                                                               hy, (const bf16*)G, ldg, M, N, K);
+                                                               hy, (const bf16*)G, ldg, gate_each, M, N, K);
   else if (x_dtype == GS_BF16 && w_dtype == GS_F32)
     heads_product_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, hx, (const float*)W, (bf16*)Y, ldy,
-                                                                hy, (const bf16*)G, ldg, M, N, K);
+                                                                hy, (const bf16*)G, ldg, gate_each, M, N, K);
   else
     GS_REQUIRE(false, "heads_product: unsupported types %d %d", x_dtype, w_dtype);
   GS_LAUNCH_CHECK("heads_product");

@@ -30,7 +30,11 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int* __restrict__
   const int P = T * top;
   for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
   __syncthreads();
-  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&counts[table[(size_t)ids[p / top] * top + p % top]], 1);
+  // (without ids the table holds the choices of the step's own rows; an entry that names no expert takes no place)
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = ids ? table[(size_t)ids[p / top] * top + p % top] : table[p];
+    if (e < E) atomicAdd(&counts[e], 1);
+  }
   __syncthreads();
   if (threadIdx.x == 0) {
     int at = 0, nt = 0;
@@ -52,14 +56,18 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int* __restrict__
   }
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
-    const int e = table[(size_t)ids[p / top] * top + p % top];
+    const int e = ids ? table[(size_t)ids[p / top] * top + p % top] : table[p];
+    if (e >= E) {
+      place_of[p] = -1;
+      continue;
+    }
     const int place = starts[e] + atomicAdd(&counts[e], 1);
     perm[place] = p / top;
     place_of[p] = place;
   }
 }
 
-// EPI 0: float32 out.  EPI 2: relu(bfloat16(v))^2, bfloat16 out.
+// EPI 0: float32 out.  EPI 1: bfloat16 out.  EPI 2: relu(bfloat16(v))^2, bfloat16 out.
 template <int EPI, typename TOut>
 __global__ __launch_bounds__(256) void moe_group_gemm_kernel(const bf16* __restrict__ X, int ldx,
                                                              const int* __restrict__ gather,
@@ -224,7 +232,7 @@ extern "C" int gs_moe_group_gemm(const void* X, int ldx, const int* gather, cons
   GS_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && max_tiles > 0 && max_tiles <= (1 << 30), "moe_group_gemm: bad sizes N=%d K=%d (K a multiple of 8)", N, K);
   GS_REQUIRE(ldx >= K && ldx % 8 == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0 && ldy >= N,
              "moe_group_gemm: X and W 16-byte aligned, row strides %d, %d", ldx, ldy);
-  GS_REQUIRE((epilogue == 0 && y_dtype == GS_F32) || (epilogue == 2 && y_dtype == GS_BF16), "moe_group_gemm: epilogue %d with output type %d", epilogue, y_dtype);
+  GS_REQUIRE((epilogue == 0 && y_dtype == GS_F32) || ((epilogue == 1 || epilogue == 2) && y_dtype == GS_BF16), "moe_group_gemm: epilogue %d with output type %d", epilogue, y_dtype);
   GS_REQUIRE(gs_ceil_div(N, MG_BN) <= 65535, "moe_group_gemm: N=%d too wide", N);
   const size_t lds = (size_t)2 * (MG_BM + MG_BN) * MG_LDR * sizeof(uint16_t);
   dim3 grid(max_tiles, gs_ceil_div(N, MG_BN));
@@ -234,6 +242,12 @@ extern "C" int gs_moe_group_gemm(const void* X, int ldx, const int* gather, cons
     (void)asked;
     moe_group_gemm_kernel<0, float><<<grid, 256, lds, stream>>>((const bf16*)X, ldx, gather, (const bf16*)W, (float*)Y, ldy,
                                                                tiles, max_tiles, n_tiles, N, K);
+  } else if (epilogue == 1) {
+    static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_group_gemm_kernel<1, bf16>),
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    (void)asked;
+    moe_group_gemm_kernel<1, bf16><<<grid, 256, lds, stream>>>((const bf16*)X, ldx, gather, (const bf16*)W, (bf16*)Y, ldy,
+                                                              tiles, max_tiles, n_tiles, N, K);
   } else {
     static const hipError_t asked = hipFuncSetAttribute(reinterpret_cast<const void*>(&moe_group_gemm_kernel<2, bf16>),
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -1127,9 +1127,10 @@ def latent_q_rot(q, H, n, r, c, cos, sin, positions, qa) -> None:
                                  _stream()))
 
 
-def heads_product(x, hx: int, w, y, hy: int, K: int, gate=None) -> torch.Tensor:
+def heads_product(x, hx: int, w, y, hy: int, K: int, gate=None, gate_each: bool = False) -> torch.Tensor:
     """``y[t, h hy : h hy + N] = w[h] @ x[t, h hx : h hx + K]`` for every head ``h`` of ``w (H, N, K)``, float32 sums in
-    a fixed order; with ``gate (T, >= H)`` the result of head ``h`` is multiplied by ``sigmoid(gate[t, h])``."""
+    a fixed order; with ``gate (T, >= H)`` the result of head ``h`` is multiplied by ``sigmoid(gate[t, h])``, with
+    ``gate_each`` and ``gate (T, >= H N)`` output ``n`` of head ``h`` by ``sigmoid(gate[t, h N + n])``."""
     _need(x.is_cuda and y.is_cuda and w.is_cuda and w.is_contiguous() and x.dim() == 2 and y.dim() == 2
           and x.stride(1) == 1 and y.stride(1) == 1, "heads_product: rows with unit column stride, on the GPU")
     H, N, Kw = w.shape
@@ -1137,11 +1138,13 @@ def heads_product(x, hx: int, w, y, hy: int, K: int, gate=None) -> torch.Tensor:
     M = x.shape[0]
     ldg = 0
     if gate is not None:
-        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == M and gate.shape[1] >= H
-              and gate.dtype == x.dtype, "heads_product: the gate is (T, >= H) of the rows' type")
+        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] == M
+              and gate.shape[1] >= (H * N if gate_each else H) and gate.dtype == x.dtype,
+              "heads_product: the gate is (T, >= H), or (T, >= H N) with a gate each, of the rows' type")
         ldg = gate.stride(0) if M > 1 else gate.shape[1]
     _check(lib().gs_heads_product(_p(x), _dt(x), x.stride(0) if M > 1 else x.shape[1], hx, _p(w), _dt(w), _p(y),
-                                  y.stride(0) if M > 1 else y.shape[1], hy, _p(gate), ldg, M, N, K, H, _stream()))
+                                  y.stride(0) if M > 1 else y.shape[1], hy, _p(gate), ldg, 1 if gate_each else 0, M, N, K,
+                                  H, _stream()))
     return y
 
 
@@ -1298,4 +1301,191 @@ def moe_table_grouped(x, ids, table, up, down, shared=None, gate=None) -> torch.
     _check(L.gs_moe_group_gemm(_p(inner), F, None, _p(down), _p(ys), F32, H, _p(tiles), max_tiles, _p(n_tiles), H, F, 0, s))
     _check(L.gs_moe_combine(_p(ys), _p(place_of), top, _p(shared), _p(gate) if shared is not None else None, ldg, _p(y),
                             _dt(y), T, H, s))
+    return y
+
+
+# ---------------------------------------------------------------------- norms in parts, convolutions over time
+
+def _cols(x, what: str):
+    """Row stride of ``x (T, C)``, which may be a range of columns of wider rows."""
+    _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1, f"{what}: rows (T, C) with unit column stride, on the GPU")
+    return x.stride(0) if x.shape[0] > 1 else max(x.shape[1], x.stride(0))
+
+
+def add_group_rmsnorm(res, d1, d2, weight, eps: float, groups: int, out_dtype, rows=None) -> torch.Tensor:
+    """``res += d1 + d2`` (each where given; not written back when ``rows`` are gathered), then every row cut into
+    ``groups`` equal parts, each divided by its own root mean square, times ``weight``.  ``rows``: int32 indices of the
+    rows to norm (None: all)."""
+    _dev(res, d1, d2, weight, rows)
+    _need(res.dtype == torch.float32 and res.dim() == 2, "add_group_rmsnorm: the residual stream is float32 (T, H)")
+    T, H = res.shape
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "add_group_rmsnorm: the weight must be float32 (H,)")
+    _need(groups >= 1 and H % groups == 0, f"add_group_rmsnorm: {groups} parts do not divide rows of {H}")
+    ds = [d for d in (d1, d2) if d is not None]
+    for d in ds:
+        _need(d.shape == res.shape and d.dtype == ds[0].dtype, "add_group_rmsnorm: deltas have the stream's shape and one type")
+    n_out = T
+    if rows is not None:
+        _i32(rows, what="rows")
+        n_out = rows.numel()
+    out = torch.empty((n_out, H), dtype=out_dtype, device=res.device)
+    _check(lib().gs_add_group_rmsnorm(_p(res), _p(ds[0]) if ds else None, _p(ds[1]) if len(ds) > 1 else None,
+                                      _dt(ds[0]) if ds else _dt(out), _p(weight), float(eps), groups, _p(out), _dt(out),
+                                      _p(rows), n_out, H, _stream()))
+    return out
+
+
+def gated_group_norm(y, z, weight, eps: float, groups: int, out_dtype) -> torch.Tensor:
+    """``y (T, H)`` float32 times ``silu(z)`` (``z (T, H)``, possibly a range of columns of wider rows), then the norm in
+    ``groups`` equal parts, times ``weight``.  float32 arithmetic; the result in ``out_dtype`` (the type of ``z``)."""
+    _dev(y, weight)
+    T, H = y.shape
+    _need(y.dtype == torch.float32 and z.shape == (T, H) and z.dtype == out_dtype, "gated_group_norm: y is float32 (T, H), z (T, H) in the result's type")
+    _need(weight.dtype == torch.float32 and weight.shape == (H,), "gated_group_norm: the weight must be float32 (H,)")
+    _need(groups >= 1 and H % groups == 0, f"gated_group_norm: {groups} parts do not divide rows of {H}")
+    ldz = _cols(z, "gated_group_norm")
+    out = torch.empty((T, H), dtype=out_dtype, device=y.device)
+    _check(lib().gs_gated_group_norm(_p(y), _p(z), _dt(z), ldz, _p(weight), float(eps), groups, _p(out), _dt(out), T, H,
+                                     _stream()))
+    return out
+
+
+def channel_conv(x, taps, bias, state, seq_of_token, q_start, slots, nseq: int, all_single: bool, out_dtype,
+                 activation=None, residual: bool = False) -> torch.Tensor:
+    """A causal convolution over time per channel, ``y_t = act(bias + sum_j taps[:, j] x_(t - K + 1 + j)) (+ x_t)``, over
+    the step's sequence portions.  ``x (T, C)`` may be a range of columns of wider rows; ``taps (C, K)`` and ``bias (C,)``
+    float32; ``state (slots, K - 1, C)`` float32 holds each request's last ``K - 1`` inputs and is moved on."""
+    _dev(taps, bias, state, seq_of_token, q_start, slots)
+    ldx = _cols(x, "channel_conv")
+    T, C = x.shape
+    K = taps.shape[1]
+    _need(taps.dtype == torch.float32 and taps.shape == (C, K), "channel_conv: taps must be float32 (C, K)")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (C,)), "channel_conv: the bias must be float32 (C,)")
+    _need(state.dtype == torch.float32 and state.dim() == 3 and (state.shape[1:] == (K - 1, C) or K == 1),
+          "channel_conv: the state must be float32 (slots, K - 1, C)")
+    _need(activation in _ACTS, f"channel_conv: activation is None or 'silu', not {activation!r}")
+    _i32(seq_of_token, T, "seq_of_token")
+    _i32(q_start, nseq + 1, "q_start")
+    _i32(slots, nseq, "slots")
+    out = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    _check(lib().gs_channel_conv(_p(x), _dt(x), ldx, _p(taps), _p(bias), _p(state), _p(seq_of_token), _p(q_start),
+                                 _p(slots), _p(out), _dt(out), C, T, nseq, C, K, _ACTS[activation], 1 if residual else 0,
+                                 1 if all_single else 0, _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- a state-space recurrence
+
+def ssd_max_state() -> int:
+    return int(lib().gs_ssd_max_state())
+
+
+def ssd_scan(xbc, rows, odt: int, dt_bias, a_log, d_skip, state, q_start, slots, nseq: int, H: int, P: int, N: int,
+             G: int) -> torch.Tensor:
+    """Per sequence and head ``h`` (group ``h // (H / G)``): ``dt = softplus(d + dt_bias[h])``,
+    ``S <- exp(-exp(a_log[h]) dt) S + dt B x^T``, ``y = S^T C + d_skip[h] x``.  ``xbc (T, H P + 2 G N)`` float32 holds
+    x, B and C side by side; ``d`` stands in ``rows (T, ld)`` from column ``odt`` on; ``state (slots, H, N, P)`` float32
+    is read and advanced.  Token by token, float32; returns ``(T, H P)`` float32."""
+    _dev(xbc, rows, dt_bias, a_log, d_skip, state, q_start, slots)
+    T = xbc.shape[0]
+    _need(xbc.dtype == torch.float32 and xbc.shape == (T, H * P + 2 * G * N), "ssd_scan: x | B | C rows must be float32 (T, H P + 2 G N)")
+    _need(rows.dim() == 2 and rows.shape[0] == T and odt + H <= rows.shape[1], "ssd_scan: the step sizes do not fit their rows")
+    for v in (dt_bias, a_log, d_skip):
+        _need(v.dtype == torch.float32 and v.shape == (H,), "ssd_scan: dt_bias, a_log and d_skip must be float32 (H,)")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.shape[1:] == (H, N, P), "ssd_scan: the state must be float32 (slots, H, N, P)")
+    _i32(q_start, nseq + 1, "q_start")
+    _i32(slots, nseq, "slots")
+    out = torch.empty((T, H * P), dtype=torch.float32, device=xbc.device)
+    _check(lib().gs_ssd_scan(_p(xbc), xbc.shape[1], H * P, H * P + G * N, _p(rows), _dt(rows), rows.shape[1], odt,
+                             _p(dt_bias), _p(a_log), _p(d_skip), _p(state), _p(q_start), _p(slots), _p(out), nseq, H, P, N,
+                             G, _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- feed-forwards chosen by a router
+
+def moe_router(x, router, correction, top: int):
+    """Scores = softmax of ``router (EA, H) @ x[t]`` in float32; the ``top`` outputs with the largest score +
+    ``correction`` are chosen (of equal ones the lowest index), their weights are their scores divided by the chosen
+    scores' sum (+ 1e-20).  Returns ``(choice int32 (T, top), weight float32 (T, top))``."""
+    _dev(router, correction)
+    ldx = _cols(x, "moe_router")
+    T, H = x.shape
+    EA = router.shape[0]
+    _need(router.shape == (EA, H) and 1 <= top <= EA, "moe_router: the router is (outputs, H), top within its outputs")
+    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (EA,)), "moe_router: the correction must be float32 (outputs,)")
+    choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    _check(lib().gs_moe_router(_p(x), _dt(x), ldx, _p(router), _dt(router), _p(correction), top, EA, H, _p(choice),
+                               _p(weight), T, _stream()))
+    return choice, weight
+
+
+def clamped_glu(gu, limit: float, alpha: float, out_dtype) -> torch.Tensor:
+    """``gu (rows, 2F)`` = gate | up  ->  ``g sigmoid(alpha g) (u + 1)`` with ``g = min(gate, limit)``,
+    ``u = clamp(up, -limit, limit)``: ``(rows, F)`` in ``out_dtype``, float32 arithmetic."""
+    _dev(gu)
+    _need(gu.dim() == 2 and gu.shape[1] % 2 == 0, "clamped_glu: rows hold gate and up side by side")
+    R, F2 = gu.shape
+    out = torch.empty((R, F2 // 2), dtype=out_dtype, device=gu.device)
+    _check(lib().gs_clamped_glu(_p(gu), _dt(gu), _p(out), _dt(out), R, F2 // 2, float(limit), float(alpha), _stream()))
+    return out
+
+
+def _routed_operands(x, choice, weight, gate_up, down, shared, what):
+    _dev(choice, weight, gate_up, down, shared)
+    ldx = _cols(x, what)
+    T, H = x.shape
+    _need(down.dim() == 3 and gate_up.dim() == 3, f"{what}: gate_up is (E, 2F, H), down (E, H, F)")
+    E, Hd, F = down.shape
+    _need(Hd == H and gate_up.shape == (E, 2 * F, H) and gate_up.dtype == down.dtype, f"{what}: gate_up is (E, 2F, H), down (E, H, F)")
+    _need(choice.dtype == torch.int32 and choice.dim() == 2 and choice.shape[0] == T and weight.dtype == torch.float32
+          and weight.shape == choice.shape, f"{what}: choices int32 (T, top) with float32 weights")
+    _need(shared is None or (shared.shape == (T, H) and shared.dtype == x.dtype), f"{what}: the shared expert's rows are (T, H) of the rows' type")
+    return ldx, T, H, E, F, choice.shape[1]
+
+
+def moe_routed(x, choice, weight, gate_up, down, limit: float, alpha: float, shared=None) -> torch.Tensor:
+    """``y[t] = sum_k weight[t, k] * expert(choice[t, k])(x[t]) (+ shared[t])``, token by token: only the chosen experts'
+    weights are read.  A choice ``>= E`` names no weights: that expert gives back ``x[t]``.  ``gate_up (E, 2F, H)`` holds
+    each expert's gate rows, then its up rows; ``down (E, H, F)``."""
+    ldx, T, H, E, F, top = _routed_operands(x, choice, weight, gate_up, down, shared, "moe_routed")
+    a = torch.empty((T, top, max(F, 1)), dtype=x.dtype, device=x.device)
+    y = torch.empty((T, H), dtype=x.dtype, device=x.device)
+    _check(lib().gs_moe_routed_up(_p(x), _dt(x), ldx, _p(choice), top, E, _p(gate_up), _dt(gate_up), F, H, float(limit),
+                                  float(alpha), _p(a), T, _stream()))
+    _check(lib().gs_moe_routed_down(_p(a), _dt(a), _p(x), ldx, _p(choice), _p(weight), top, E, _p(down), _dt(down), F, H,
+                                    _p(shared), _p(y), T, _stream()))
+    return y
+
+
+def moe_routed_grouped_ok(x, gate_up, down) -> bool:
+    """Whether :func:`moe_routed_grouped` takes these operands: bfloat16 throughout, widths in whole 16-byte pieces."""
+    bf = torch.bfloat16
+    return (x.dtype is bf and gate_up.dtype is bf and down.dtype is bf and x.dim() == 2 and x.stride(1) == 1
+            and x.shape[1] % 8 == 0 and down.shape[2] % 8 == 0 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0)
+            and x.data_ptr() % 16 == 0 and 0 < down.shape[0] <= 4096)
+
+
+def moe_routed_grouped(x, choice, weight, gate_up, down, limit: float, alpha: float, shared=None) -> torch.Tensor:
+    """:func:`moe_routed` for steps of many tokens (bfloat16): the (token, choice) pairs are sorted by expert on the
+    device and every expert's weights are read once, by products on the matrix cores over its pairs' rows."""
+    _need(moe_routed_grouped_ok(x, gate_up, down), "moe_routed_grouped: bfloat16 rows and weights, widths multiples of 8")
+    ldx, T, H, E, F, top = _routed_operands(x, choice, weight, gate_up, down, shared, "moe_routed_grouped")
+    P = T * top
+    dev = x.device
+    max_tiles = -(-P // lib().gs_moe_group_rows()) + E
+    index = torch.empty(2 * P + 3 * max_tiles + 1, dtype=torch.int32, device=dev)
+    perm, place_of, tiles, n_tiles = index[:P], index[P:2 * P], index[2 * P:2 * P + 3 * max_tiles], index[2 * P + 3 * max_tiles:]
+    gu = torch.empty((P, 2 * F), dtype=torch.bfloat16, device=dev)
+    ys = torch.empty((P, H), dtype=torch.float32, device=dev)
+    y = torch.empty((T, H), dtype=x.dtype, device=dev)
+    s = _stream()
+    L = lib()
+    _check(L.gs_moe_route(None, _p(choice), T, top, E, _p(perm), _p(place_of), _p(tiles), max_tiles, _p(n_tiles), s))
+    _check(L.gs_moe_group_gemm(_p(x), ldx, _p(perm), _p(gate_up), _p(gu), BF16, 2 * F, _p(tiles), max_tiles, _p(n_tiles),
+                               2 * F, H, 1, s))
+    inner = clamped_glu(gu, limit, alpha, torch.bfloat16)
+    _check(L.gs_moe_group_gemm(_p(inner), F, None, _p(down), _p(ys), F32, H, _p(tiles), max_tiles, _p(n_tiles), H, F, 0, s))
+    _check(L.gs_moe_routed_combine(_p(ys), _p(place_of), _p(weight), top, _p(x), ldx, _p(shared), _p(y), _dt(y), T, H, s))
     return y

@@ -13,7 +13,7 @@ import torch
 
 from ..config.spec import ModelSpec
 from ..errors import ConfigError
-from ..parts.base import MATRIX, TABLE, TensorSpec
+from ..parts.base import MATRIX, TABLE, VECTOR, TensorSpec
 from ..parts.registry import build, part_class
 from ..parts.rmsnorm import ResidualStream, row_weight_of
 
@@ -35,6 +35,9 @@ def tensor_table(spec: ModelSpec) -> Dict[str, TensorSpec]:
             put(spec.names["embed_norm." + local], ts)
     if not spec.tie_embeddings:
         put(spec.names["head"], TensorSpec((spec.vocab, spec.hidden), MATRIX))
+    if spec.reentry is not None:
+        put(spec.names["reentry.weight"], TensorSpec((spec.hidden, 2 * spec.hidden), MATRIX))
+        put(spec.names["reentry.step"], TensorSpec((len(spec.reentry.at), spec.hidden), VECTOR))
     for i, b in enumerate(spec.blocks):
         for local, ts in part_class("block", b).tensor_specs(b).items():
             if local not in b.names:
@@ -59,6 +62,7 @@ class Model:
         self.embed_norm = build("norm", spec.embed_norm, rt) if spec.embed_norm is not None else None
         self.embed = None
         self.head = None
+        self.reentry_weight = self.reentry_step = None
 
     def cache_needs(self) -> List[Optional[object]]:
         """For each entry of the schedule: what its own cache must hold (None: none, or it reads another's)."""
@@ -78,6 +82,9 @@ class Model:
         if self.embed_norm is not None:
             self.embed_norm.bind({k: tensors[s.names["embed_norm." + k]]
                                   for k in part_class("norm", s.embed_norm).tensor_specs(s.embed_norm)})
+        if s.reentry is not None:
+            self.reentry_weight = self.rt.prepare(tensors[s.names["reentry.weight"]])
+            self.reentry_step = tensors[s.names["reentry.step"]].contiguous()
         for b, block in zip(s.blocks, self.blocks):
             local = {k: tensors[b.names[k]] for k in part_class("block", b).tensor_specs(b)}
             block.bind(local)
@@ -106,10 +113,29 @@ class Model:
         scale = 1.0 if self.spec.embed_scale is None else float(self.spec.embed_scale)
         with rt.stage("embed"):
             stream = self._embed(ctx, order, scale)
+        reentries = {} if self.spec.reentry is None else {at: t for t, at in enumerate(self.spec.reentry.at)}
+        # the embedding output, kept for every re-entry of this step (in the activation type: it is a product's operand
+        # from here on)
+        x0 = stream.res.to(rt.dtype, copy=True) if reentries else None
         for i, call in enumerate(self.spec.schedule):
+            if i in reentries:
+                with rt.stage("reentry"):
+                    stream = self._reenter(stream, x0, reentries[i])
             stream.following = readers[i]
             order[i].forward(stream, ctx, ctx.cache_view(i))
         return stream
+
+    def _reenter(self, stream: ResidualStream, x0, t: int) -> ResidualStream:
+        """``x <- W [x; x0] + step[t]``: the stream and the embedding output side by side through one product, float32
+        sums, the pass's vector added in float32; the result is the new stream."""
+        rt = self.rt
+        stream.flush(rt)
+        T, W = stream.res.shape
+        rows = torch.empty((T, 2 * W), dtype=rt.dtype, device=stream.res.device)
+        rows[:, :W].copy_(stream.res)
+        rows[:, W:].copy_(x0)
+        y = rt.linear(rows, self.reentry_weight, out_dtype=torch.float32)
+        return ResidualStream(rt.ops.add_bias(y, self.reentry_step[t], torch.float32, out=y))
 
     def logits(self, stream: ResidualStream, rows) -> torch.Tensor:
         """The final norm of the stream's ``rows`` (int32 on the device; None: all, in order) and the head: float32."""

@@ -153,6 +153,95 @@ class ParallelBlock(PreNormBlock):
         return False
 
 
+class SharedNormBlock(Part):
+    """``h += mixer(a + conv(a)) + ffn(a)`` with ``a = norm(h)``: one norm, read by both sub-layers; the mixer's input
+    may get a causal convolution over time added to it (``spec.input_taps``), whose last inputs are the request's state,
+    kept in its slot beside whatever the mixer keeps.  The norm's pass adds the two results that the block before left;
+    this block's own two results stay beside the stream for whoever norms it next."""
+
+    def __init__(self, spec, rt):
+        super().__init__(spec, rt)
+        self.norm = build("norm", spec.norm, rt)
+        self.mixer = build("mixer", spec.mixer, rt)
+        self.ffn = build("ffn", spec.ffn, rt) if spec.ffn is not None else None
+        self.taps = None
+
+    @staticmethod
+    def _width(spec) -> int:
+        return int(spec.norm.size)
+
+    @staticmethod
+    def tensor_specs(spec):
+        from .base import VECTOR, TensorSpec
+        out = {}
+        roles = [("norm", "norm", spec.norm), ("mixer", "mixer", spec.mixer)]
+        if spec.ffn is not None:
+            roles.append(("ffn", "ffn", spec.ffn))
+        for role, category, sub in roles:
+            for name, ts in part_class(category, sub).tensor_specs(sub).items():
+                out[f"{role}.{name}"] = ts
+        if spec.input_taps is not None:
+            out["input_conv.weight"] = TensorSpec((SharedNormBlock._width(spec), spec.input_taps), VECTOR)
+        return out
+
+    @staticmethod
+    def _mixer_needs(spec) -> tuple:
+        cls = part_class("mixer", spec.mixer)
+        need = cls.cache_need(spec.mixer) if hasattr(cls, "cache_need") else None
+        return tuple(need) if isinstance(need, (tuple, list)) else (need,)
+
+    @staticmethod
+    def cache_need(spec):
+        from .base import SlotState
+        mixer = SharedNormBlock._mixer_needs(spec)
+        if spec.input_taps is None:
+            return mixer if len(mixer) > 1 else mixer[0]
+        # (a single tap has no history; a row is kept all the same, which nobody reads)
+        own = SlotState((("input_history", (max(spec.input_taps - 1, 1), SharedNormBlock._width(spec)), "float32"),))
+        return (own,) + mixer
+
+    def bind(self, tensors):
+        self.norm.bind(sub_tensors(tensors, "norm"))
+        self.mixer.bind(sub_tensors(tensors, "mixer"))
+        if self.ffn is not None:
+            self.ffn.bind(sub_tensors(tensors, "ffn"))
+        if self.spec.input_taps is not None:
+            self.taps = tensors["input_conv.weight"].contiguous()
+
+    @property
+    def first_norm(self):
+        return None                 # the norm's pass is the block's own business
+
+    def forward(self, stream, ctx, cache):
+        rt, ops, s = self.rt, self.rt.ops, self.spec
+        with rt.stage("norm"):
+            a = self.norm.add_norm(stream)
+        x = a
+        mixer_cache = cache
+        if s.input_taps is not None:
+            with rt.stage("input_conv"):
+                history = cache[0].state["input_history"]
+                rest = cache[1:]
+                mixer_cache = rest if len(rest) > 1 else rest[0]
+                x = ops.channel_conv(a, self.taps, None, history, ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq,
+                                     ctx.all_single, rt.dtype, residual=True)
+        with rt.stage(getattr(self.mixer, "stage", "mixer")):
+            m = rt.dense(self.mixer.forward(x, ctx, mixer_cache))
+        f = None
+        if self.ffn is not None:
+            with rt.stage(getattr(self.ffn, "stage", "ffn")):
+                f = rt.dense(self.ffn.forward(a, ctx))
+        stream.pending = (m, f)
+
+    @property
+    def graph_safe(self) -> bool:
+        parts = [self.norm, self.mixer] + ([self.ffn] if self.ffn is not None else [])
+        return all(getattr(p, "graph_safe", False) for p in parts)
+
+    portions_recordable = False
+
+
 register("block", "prenorm", PreNormBlock)
+register("block", "shared_norm", SharedNormBlock)
 register("block", "parallel", ParallelBlock)
 register("block", "outnorm", OutNormBlock)

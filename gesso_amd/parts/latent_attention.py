@@ -43,8 +43,13 @@ class LatentAttention(Part):
         if spec.rot_dim % 2:
             raise ValueError("rotated features come in pairs")
         self.position = build("position", spec.position, rt)
-        if spec.rot_dim and (self.position.rotary_dim != spec.rot_dim or getattr(self.position, "layout", "half") != "half"):
-            raise ValueError("the rotated part of a head is rotated whole, in half-split pairs")
+        if spec.rot_dim and self.position.rotary_dim != spec.rot_dim:
+            raise ValueError("the rotated part of a head is rotated whole")
+        # The kernels turn half-split pairs (i, i + r/2).  An encoding whose pairs are neighbours (2i, 2i + 1) is served
+        # by reordering, at load, the rows of the two products that make the rotated features (evens first, then odds):
+        # queries and the shared key part are reordered alike, so every score is the same sum in another order, and
+        # nobody else reads these features (the cache holds the key part in the kernels' order).
+        self.reorder = bool(spec.rot_dim) and getattr(self.position, "layout", "half") == "interleaved"
 
     @staticmethod
     def tensor_specs(spec):
@@ -54,7 +59,7 @@ class LatentAttention(Part):
                "kv_norm.weight": TensorSpec((c,), VECTOR, "one_plus_normal"), "k_up.weight": TensorSpec((H * n, c), MATRIX),
                "v_up.weight": TensorSpec((H * dv, c), MATRIX), "out.weight": TensorSpec((W, H * dv), MATRIX)}
         if spec.gated:
-            out["gate.weight"] = TensorSpec((H, W), MATRIX)
+            out["gate.weight"] = TensorSpec((H * dv if getattr(spec, "gate_each", False) else H, W), MATRIX)
         return out
 
     @staticmethod
@@ -63,13 +68,20 @@ class LatentAttention(Part):
 
     def bind(self, tensors):
         s, rt = self.spec, self.rt
-        H, n, dv, c = s.n_heads, s.plain_dim, s.value_dim, s.kv_rank
-        ws = [tensors["q_down.weight"], tensors["kv_down.weight"]] + ([tensors["gate.weight"]] if s.gated else [])
+        H, n, r, dv, c = s.n_heads, s.plain_dim, s.rot_dim, s.value_dim, s.kv_rank
+        w_dkv, w_uq = tensors["kv_down.weight"], tensors["q_up.weight"]
+        if self.reorder:
+            order = torch.cat([torch.arange(0, r, 2), torch.arange(1, r, 2)]).to(w_dkv.device)
+            w_dkv = torch.cat([w_dkv[:c], w_dkv[c:][order]], 0)
+            per_head = torch.cat([torch.arange(n, device=order.device), n + order])
+            rows = (torch.arange(H, device=order.device)[:, None] * (n + r) + per_head[None, :]).reshape(-1)
+            w_uq = w_uq[rows].contiguous()
+        ws = [tensors["q_down.weight"], w_dkv] + ([tensors["gate.weight"]] if s.gated else [])
         if len({w.dtype for w in ws}) > 1:
             ws = [w.float() for w in ws]
         self.w_in = rt.prepare(_pad_rows(torch.cat(ws, 0)))
         self.q_norm, self.kv_norm = tensors["q_norm.weight"], tensors["kv_norm.weight"]
-        self.w_uq = rt.prepare(tensors["q_up.weight"])
+        self.w_uq = rt.prepare(w_uq)
         # W_uk[h]^T as the weight of a per-head product: (H, c, n); W_uv[h]: (H, dv, c)
         self.uk_t = tensors["k_up.weight"].reshape(H, n, c).transpose(1, 2).contiguous() if n else None
         self.uv = tensors["v_up.weight"].reshape(H, dv, c).contiguous()
@@ -92,7 +104,8 @@ class LatentAttention(Part):
         with rt.stage("attn_core"):
             mixed = self.attend(qa, ctx, cache)
         o = torch.empty((T, H * dv), dtype=mixed.dtype, device=mixed.device)
-        ops.heads_product(mixed, c, self.uv, o, dv, c, gate=down[:, qr + c + r:] if s.gated else None)
+        ops.heads_product(mixed, c, self.uv, o, dv, c, gate=down[:, qr + c + r:] if s.gated else None,
+                          gate_each=bool(s.gated and getattr(s, "gate_each", False)))
         return rt.linear(o, self.w_out)
 
     def attend(self, qa, ctx, cache) -> torch.Tensor:

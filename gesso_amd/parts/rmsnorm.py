@@ -124,4 +124,36 @@ class RMSNorm(Part):
         return y
 
 
+class GroupRMSNorm(Part):
+    """RMS norm in parts: the row is cut into ``groups`` equal consecutive parts, each divided by its own
+    ``sqrt(mean(part^2) + eps)``; then the weight.  One part: the plain norm.  float32 arithmetic."""
+
+    graph_safe = True
+
+    @staticmethod
+    def tensor_specs(spec):
+        return {"weight": TensorSpec((spec.size,), VECTOR, "one_plus_normal")}
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+
+    def add_norm(self, stream: ResidualStream, rows=None, out=None, out_dtype=None):
+        """Add what is pending to the stream (both results of a block that left two), then norm it (only ``rows`` of
+        it when given)."""
+        rt = self.rt
+        if stream.bias is not None or (rows is not None and stream.pending is not None):
+            stream.flush(rt)
+        held = stream.pending if isinstance(stream.pending, tuple) else (stream.pending, None)
+        if len(held) > 2 or len({d.dtype for d in held if d is not None}) > 1:
+            stream.flush(rt)
+            held = (None, None)
+        y = rt.ops.add_group_rmsnorm(stream.res, held[0], held[1], self.weight, self.spec.eps, self.spec.groups,
+                                     out_dtype or rt.dtype, rows=rows)
+        if rows is None or stream.pending is None:
+            stream.pending = None
+        stream.ssq = stream.xs = stream.xs_for = stream.normed = stream.rows = None
+        return y
+
+
 register("norm", "rmsnorm", RMSNorm)
+register("norm", "group_rmsnorm", GroupRMSNorm)
