@@ -61,8 +61,9 @@ def weight_bytes(engine) -> int:
         return out
 
     for b in m.blocks:
-        for part in (b.mixer_norm, b.mixer, b.ffn_norm, b.ffn):
+        for part in (getattr(b, name, None) for name in ("mixer_norm", "norm", "mixer", "ffn_norm", "ffn")):
             tensors += of(part)
+        tensors += [v for v in vars(b).values() if isinstance(v, torch.Tensor)]      # a block's own (an input convolution's taps)
     for t in tensors:
         if t.data_ptr() not in seen:
             seen.add(t.data_ptr())
@@ -444,6 +445,59 @@ def fazezen_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), o
     return out
 
 
+TOGALORN_SIZES = {
+    # the attention layers and the experts as wide as Makuzen's of that name; state-space layers twice the width inside,
+    # in heads of 64 with a state of 128 rows; six layers of which the first two run twice (eight layer runs, two
+    # re-entries of the embedding): m m | m m | a m m a
+    "1024": dict(width=1024, ssm=dict(heads=32, vdim=64, state=128, groups=1, norm_groups=1), norm_groups=2, beside="1024"),
+    "2048": dict(width=2048, ssm=dict(heads=64, vdim=64, state=128, groups=8, norm_groups=8), norm_groups=4, beside="2048"),
+}
+
+
+def togalorn_config(size: str, max_position: int = 4096):
+    from gesso_amd.config import (ExpertConfig, LatentMixerConfig, LoopConfig, Mamba2MixerConfig, MoEConfig, TogalornConfig,
+                                  TogalornLayer)
+    z = TOGALORN_SIZES[size]
+    k = MAKUZEN_SIZES[z["beside"]]
+    mlp = MoEConfig(k["experts"], k["top"], 2, ExpertConfig(k["ff"], 7.0), ExpertConfig(k["shared"], 7.0))
+    s = z["ssm"]
+    state = TogalornLayer("mamba2", Mamba2MixerConfig(s["heads"], s["vdim"], s["state"], s["groups"], s["norm_groups"], 4), mlp)
+    attn = TogalornLayer("latent_attention", LatentMixerConfig(k["heads"], k["dim"], k["rot"], k["vdim"], k["q_rank"], k["kv_rank"],
+                                                               (k["dim"] + k["rot"]) ** -0.5, 1e6), mlp)
+    return TogalornConfig(vocab=k["vocab"], width=z["width"], layers=(state, state, attn, state, state, attn), norm_eps=1e-6,
+                          norm_groups=z["norm_groups"], embedding_scale=float(z["width"]) ** 0.5, canon_taps=4,
+                          loop=LoopConfig(0, 2, 2), max_position=max_position)
+
+
+def togalorn_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), only: str = "", batches=(8, 64)) -> dict:
+    """Togalorn (state-space layers and latent attention behind one norm in parts, experts chosen by a softmax router, a
+    run of layers passed twice) at two sets of layer sizes, beside Makuzen of the same width and as many layer runs: a
+    2,048-token prompt in one step, and decode steps at 512-token prompts."""
+    from gesso_amd import Engine
+    from gesso_amd.parts import RuntimeOptions
+    out = {"metric": "Togalorn beside Makuzen at equal width and depth: prefill and decode tok/s", "unit": "tok/s", "dtype": "bf16",
+           "data": "synthetic: uniform random token ids, random weights N(0, 0.02)", "sizes": {}}
+    for size in sizes:
+        row = {}
+        for name, cfg in (("togalorn", togalorn_config(size)), ("makuzen", makuzen_config(TOGALORN_SIZES[size]["beside"]))):
+            if only and only != name:
+                continue
+            engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=4096,
+                                        max_tokens=max(batches) * (512 + steps + warmup + 32) + 4096, num_slots=max(batches) + 1,
+                                        options=RuntimeOptions(tune_library=True))
+            sec = prefill_run(engine, cfg, 2048)
+            r = {"prefill_tok_s": round(2048 / sec, 1), "prefill_ms": round(sec * 1e3, 3), "weights_gb": round(weight_bytes(engine) / 1e9, 3)}
+            for b in batches:
+                dt, _ = decode_run(engine, cfg, b, 512, steps, warmup, seed=40 + b)
+                r[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+                r[f"decode_b{b}_ms"] = round(dt / steps * 1e3, 4)
+            row[name] = r
+            del engine
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -463,13 +517,15 @@ def main() -> int:
     ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
                     "replaying recordings of them (the prefill of the default line, --workload serve)")
     ap.add_argument("--token-budget", type=int, default=4096, help="--workload serve: the most tokens a step holds")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen", "fazezen"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen", "fazezen", "togalorn"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
                          "stages: the decode step stage by stage; makuzen: the Makuzen design at two sets of layer sizes "
                          "beside LFM2 of equal width and depth; fazezen: the same for the Fazezen design")
     ap.add_argument("--fazezen-sizes", default="1024,2048", help="--workload fazezen: which of its sizes")
     ap.add_argument("--fazezen-only", default="", choices=["", "fazezen", "lfm2"], help="--workload fazezen: one of the two models (for profiling)")
+    ap.add_argument("--togalorn-sizes", default="1024,2048", help="--workload togalorn: which of its sizes")
+    ap.add_argument("--togalorn-only", default="", choices=["", "togalorn", "makuzen"], help="--workload togalorn: one of the two models (for profiling)")
     ap.add_argument("--makuzen-sizes", default="1024,2048", help="--workload makuzen: which of its sizes")
     ap.add_argument("--makuzen-only", default="", choices=["", "makuzen", "lfm2"], help="--workload makuzen: one of the two models (for profiling)")
     args = ap.parse_args()
@@ -487,6 +543,10 @@ def main() -> int:
         if args.workload == "fazezen":
             print(json.dumps(fazezen_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.fazezen_sizes.split(",")),
                                               args.fazezen_only)))
+            return 0
+        if args.workload == "togalorn":
+            print(json.dumps(togalorn_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.togalorn_sizes.split(",")),
+                                               args.togalorn_only)))
             return 0
         if args.workload == "serve":
             print(json.dumps(serve_workload(record=not args.launched_portions, tune=not args.no_tune, budget=args.token_budget)))

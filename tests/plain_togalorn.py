@@ -181,9 +181,19 @@ def route(h, router, correction, top: int):
     return chosen, picked / (picked.sum(-1, keepdim=True) + 1e-20), s
 
 
-def moe(h, w, p, m, store=_keep):
+def choice_margin(scores, correction, top: int):
+    """Per token: by how much the last chosen output's corrected score leads the best one left out (inf: all chosen)."""
+    ranked = torch.sort(scores + correction, dim=-1, descending=True).values
+    if top >= ranked.shape[1]:
+        return torch.full((ranked.shape[0],), math.inf, dtype=ranked.dtype)
+    return ranked[:, top - 1] - ranked[:, top]
+
+
+def moe(h, w, p, m, store=_keep, margins=None):
     E, top = m["router"]["experts"], m["router"]["top"]
-    chosen, weights, _ = route(h, w[p + ".router"], w[p + ".correction"], top)
+    chosen, weights, scores = route(h, w[p + ".router"], w[p + ".correction"], top)
+    if margins is not None:
+        margins.append(choice_margin(scores, w[p + ".correction"], top))
     y = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, a in zip(chosen[t].tolist(), weights[t]):
@@ -200,7 +210,7 @@ def moe(h, w, p, m, store=_keep):
 
 # --------------------------------------------------------------------------- layers, the model
 
-def layer(x, w, i, cfg, positions, store=_keep):
+def layer(x, w, i, cfg, positions, store=_keep, margins=None):
     """``x + mixer(a + conv(a)) + ff(a)`` with ``a`` the norm in parts of ``x``."""
     L = cfg["layers"][i]
     eps, groups = float(cfg["norm"]["eps"]), int(cfg["norm"].get("groups") or 1)
@@ -215,7 +225,7 @@ def layer(x, w, i, cfg, positions, store=_keep):
     else:
         raise ValueError(f"unknown layer type {L['type']!r}")
     if L.get("mlp") is not None:
-        y = y + moe(a, w, f"l{i}.mlp", L["mlp"], store)
+        y = y + moe(a, w, f"l{i}.mlp", L["mlp"], store, margins)
     return x + y
 
 
@@ -248,9 +258,10 @@ def read_weights(model_dir: str, dtype=torch.float64) -> dict:
     return out
 
 
-def forward(cfg: dict, w: dict, ids, store=_keep, layers_out=None) -> torch.Tensor:
+def forward(cfg: dict, w: dict, ids, store=_keep, layers_out=None, margins=None) -> torch.Tensor:
     """Logits ``(T, vocab)`` of the whole sequence ``ids``, positions from 0.  ``layers_out``: a list that receives the
-    residual stream after every layer run."""
+    residual stream after every layer run.  ``margins``: a list that receives, for every feed-forward run, each token's
+    :func:`choice_margin`."""
     ids = [int(t) for t in ids]
     positions = list(range(len(ids)))
     x0 = embedding(w["embed"], ids, float((cfg.get("embedding") or {}).get("scale") or 1.0))
@@ -258,7 +269,7 @@ def forward(cfg: dict, w: dict, ids, store=_keep, layers_out=None) -> torch.Tens
     for i, t, first in run_order(cfg):
         if first:
             x = linear(torch.cat([store(x), store(x0)], 1), w["loop.in"]) + w["loop.step"][t]
-        x = layer(x, w, i, cfg, positions, store)
+        x = layer(x, w, i, cfg, positions, store, margins)
         if layers_out is not None:
             layers_out.append(x.clone())
     eps, groups = float(cfg["norm"]["eps"]), int(cfg["norm"].get("groups") or 1)
