@@ -79,6 +79,7 @@ class BatchContext:
             setattr(self, k, v)
         self._storage = storage
         self._tiles = None
+        self._segments = None
 
     def cache_view(self, call: int):
         return self._storage.view(call, self.block_tables)
@@ -107,6 +108,21 @@ class BatchContext:
             t = torch.tensor([seq, row, cnt], dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
             self._tiles = ((rows, skip), t)
         return self._tiles[1]
+
+    def state_segments(self, seg_len: int):
+        """The step's portions cut into segments of at most ``seg_len`` tokens, for recurrences that walk segments side by
+        side: ``(int32 on the device, number of segments)``; the tensor holds where each sequence's segments begin
+        (``nseq + 1`` entries), then a row of four per segment: sequence, first token within the portion, tokens, 1 at a
+        portion's last segment.  Made once per step, on first use."""
+        if self._segments is None or self._segments[0] != seg_len:
+            first, rows = [0], []
+            for i, n in enumerate(self.q_lens):
+                for a in range(0, max(n, 1), seg_len):
+                    rows += [i, a, max(0, min(seg_len, n - a)), 1 if a + seg_len >= n else 0]
+                first.append(len(rows) // 4)
+            t = torch.tensor(first + rows, dtype=torch.int32).pin_memory().to(self.token_ids.device, non_blocking=True)
+            self._segments = (seg_len, t, len(rows) // 4)
+        return self._segments[1], self._segments[2]
 
     def subtile_lists(self, wq: int, skip: int = 0, paired: bool = True):
         """:func:`subtile_lists` of this step's sequences from ``skip`` on, on the host."""

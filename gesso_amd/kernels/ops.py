@@ -1381,11 +1381,13 @@ def ssd_max_state() -> int:
 
 
 def ssd_scan(xbc, rows, odt: int, dt_bias, a_log, d_skip, state, q_start, slots, nseq: int, H: int, P: int, N: int,
-             G: int) -> torch.Tensor:
+             G: int, segments=None) -> torch.Tensor:
     """Per sequence and head ``h`` (group ``h // (H / G)``): ``dt = softplus(d + dt_bias[h])``,
     ``S <- exp(-exp(a_log[h]) dt) S + dt B x^T``, ``y = S^T C + d_skip[h] x``.  ``xbc (T, H P + 2 G N)`` float32 holds
     x, B and C side by side; ``d`` stands in ``rows (T, ld)`` from column ``odt`` on; ``state (slots, H, N, P)`` float32
-    is read and advanced.  Token by token, float32; returns ``(T, H P)`` float32."""
+    is read and advanced.  Token by token, float32; returns ``(T, H P)`` float32.  ``segments``: ``(table, count)`` as
+    ``BatchContext.state_segments`` makes them: the portions are then walked segment by segment side by side (three
+    launches: what each segment adds to a state, every segment's first state, the segments with their outputs)."""
     _dev(xbc, rows, dt_bias, a_log, d_skip, state, q_start, slots)
     T = xbc.shape[0]
     _need(xbc.dtype == torch.float32 and xbc.shape == (T, H * P + 2 * G * N), "ssd_scan: x | B | C rows must be float32 (T, H P + 2 G N)")
@@ -1396,6 +1398,15 @@ def ssd_scan(xbc, rows, odt: int, dt_bias, a_log, d_skip, state, q_start, slots,
     _i32(q_start, nseq + 1, "q_start")
     _i32(slots, nseq, "slots")
     out = torch.empty((T, H * P), dtype=torch.float32, device=xbc.device)
+    if segments is not None:
+        table, nsegs = segments
+        _i32(table, nseq + 1 + 4 * nsegs, "segments")
+        ws = torch.empty((nsegs * H * N * P + nsegs * H,), dtype=torch.float32, device=xbc.device)
+        _check(lib().gs_ssd_scan_segments(_p(xbc), xbc.shape[1], H * P, H * P + G * N, _p(rows), _dt(rows), rows.shape[1],
+                                          odt, _p(dt_bias), _p(a_log), _p(d_skip), _p(state), _p(q_start), _p(slots),
+                                          _p(out), nseq, H, P, N, G, table.data_ptr(), table.data_ptr() + 4 * (nseq + 1),
+                                          nsegs, ws.data_ptr(), ws.data_ptr() + 4 * nsegs * H * N * P, _stream()))
+        return out
     _check(lib().gs_ssd_scan(_p(xbc), xbc.shape[1], H * P, H * P + G * N, _p(rows), _dt(rows), rows.shape[1], odt,
                              _p(dt_bias), _p(a_log), _p(d_skip), _p(state), _p(q_start), _p(slots), _p(out), nseq, H, P, N,
                              G, _stream()))

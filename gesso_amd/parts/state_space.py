@@ -11,7 +11,9 @@ groups of heads that share their B and C:
 
 The request's state is one slot: the convolution's last ``taps - 1`` inputs and the matrices ``S``, float32 in both
 precisions, zero at a request's start.  From the convolution's output to the norm nothing is rounded to the
-activation type.
+activation type.  A portion of ``2 * SEGMENT`` tokens or more is walked in segments side by side (the state a segment
+starts from is put together from what the segments before it add); results then differ from the walk in one piece by
+float32 rounding.
 """
 from __future__ import annotations
 
@@ -19,6 +21,9 @@ import torch
 
 from .base import MATRIX, VECTOR, Part, SlotState, TensorSpec
 from .registry import register
+
+
+SEGMENT = 128      # tokens a segment: long portions are walked in segments of this many, side by side
 
 
 class StateSpace(Part):
@@ -74,8 +79,10 @@ class StateSpace(Part):
                                    ctx.seq_of_token, ctx.q_start, ctx.slots, ctx.nseq, ctx.all_single, torch.float32,
                                    activation="silu")
         with rt.stage("state_scan"):
+            # a step that brings a long portion: its segments side by side instead of one walk a sequence and head
+            segments = ctx.state_segments(SEGMENT) if ctx.max_q_len >= 2 * SEGMENT else None
             y = ops.ssd_scan(xbc, rows, inner + chan, self.dt_bias, self.a_log, self.d_skip, cache.state["state"],
-                             ctx.q_start, ctx.slots, ctx.nseq, H, P, N, G)
+                             ctx.q_start, ctx.slots, ctx.nseq, H, P, N, G, segments=segments)
         with rt.stage("state_norm"):
             g = ops.gated_group_norm(y, rows[:, :inner], self.norm_weight, s.eps, s.norm_groups, rt.dtype)
         return rt.linear(g, self.w_out)

@@ -152,9 +152,20 @@ def test_gate_then_norm_in_parts(ops, dtype, H, groups):
     assert float((other - want).abs().max()) > 10 * tol(dtype, want)
 
 
-def scan_case(ops, dtype, H, P_, N, G, lens, pieces=None, seed=0, a_log=None, meet=None):
+def segment_table(sizes, seg_len):
+    """Where each sequence's segments begin, then (sequence, first token within the portion, tokens, 1 at the last)."""
+    first, rows = [0], []
+    for i, n in enumerate(sizes):
+        for a in range(0, n, seg_len):
+            rows += [i, a, min(seg_len, n - a), 1 if a + seg_len >= n else 0]
+        first.append(len(rows) // 4)
+    return i32(first + rows), len(rows) // 4
+
+
+def scan_case(ops, dtype, H, P_, N, G, lens, pieces=None, seed=0, a_log=None, meet=None, seg_len=None):
     """Rows of x | B | C (float32, as the convolution leaves them) and of step sizes inside wider rows of ``dtype``, for
-    sequences of ``lens`` tokens fed in ``pieces`` (default: whole), states in shuffled slots.  ``meet``: ``(sequence,
+    sequences of ``lens`` tokens fed in ``pieces`` (default: whole), states in shuffled slots.  ``seg_len``: a step that
+    brings a portion of twice that many tokens is walked in segments of that many, side by side.  ``meet``: ``(sequence,
     far token, near token, head)``: the far token's B row and the near one's C row are made to meet, and the far
     token's x row and step size are made large."""
     g = gen(seed)
@@ -188,7 +199,8 @@ def scan_case(ops, dtype, H, P_, N, G, lens, pieces=None, seed=0, a_log=None, me
         rows = torch.cat([xbc[s][done[s]:done[s] + n] for s, n in zip(live, sizes)]).to(DEV)
         dr = torch.cat([drows[s][done[s]:done[s] + n] for s, n in zip(live, sizes)]).to(DEV)
         y = ops.ssd_scan(rows, dr, odt, dt_bias.to(DEV), a_log.to(DEV), d_skip.to(DEV), st, i32(starts_of(sizes)),
-                         i32([slots[s] for s in live]), len(live), H, P_, N, G)
+                         i32([slots[s] for s in live]), len(live), H, P_, N, G,
+                         segments=segment_table(sizes, seg_len) if seg_len and max(sizes) >= 2 * seg_len else None)
         at = 0
         for s, n in zip(live, sizes):
             got[s].append(y[at:at + n].cpu())
@@ -202,6 +214,7 @@ def scan_case(ops, dtype, H, P_, N, G, lens, pieces=None, seed=0, a_log=None, me
                                   x[:, inner + G * N:].reshape(n, G, N), dt, a_log.double(), d_skip.double(), H // G).reshape(n, inner))
     untouched = [s for s in range(state.shape[0]) if s not in slots]
     assert all(torch.isnan(st[s]).all() for s in untouched)
+    scan_case.states = [st[sl].cpu() for sl in slots]
     return [torch.cat(g_) for g_ in got], want, xbc, d_skip
 
 
@@ -220,15 +233,32 @@ def test_state_recurrence_over_unequal_sequences_and_any_cut(ops, dtype, H, P_, 
         assert torch.equal(cut[s], got[s]), s
 
 
-@pytest.mark.parametrize("pieces", [None, [[300] + [1] * 60], [[7] * 51 + [3]]])
-def test_a_state_keeps_what_it_was_given_hundreds_of_tokens_before(ops, pieces):
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,P_,N,G,seg", [(4, 16, 24, 2, 32), (2, 64, 64, 1, 64), (2, 128, 128, 2, 128), (5, 10, 7, 5, 16), (8, 32, 48, 2, 50)])
+def test_state_recurrence_in_segments_side_by_side(ops, dtype, H, P_, N, G, seg):
+    """Long portions beside short ones and single tokens; a portion that ends on a segment's edge, one a token past it;
+    states that go on from earlier steps, in segments again and token by token."""
+    lens = [1, 2 * seg, 40, 4 * seg + 1, 2, 3 * seg + seg // 2 + 7]
+    whole, want, _, _ = scan_case(ops, dtype, H, P_, N, G, lens, seed=H + N)
+    states = scan_case.states
+    for pieces in (None, [[1], [2 * seg], [20, 1, 19], [2 * seg + 3, 1, 1, 2 * seg - 4], [1, 1], [seg + 7, 2 * seg + seg // 2]]):
+        got, _, _, _ = scan_case(ops, dtype, H, P_, N, G, lens, pieces, seed=H + N, seg_len=seg)
+        for s in range(len(lens)):
+            bound = 5e-5 * max(1.0, float(want[s].abs().max()))
+            assert float((got[s].double() - want[s]).abs().max()) <= bound, s
+            assert float((got[s] - whole[s]).abs().max()) <= bound, s
+            assert float((scan_case.states[s] - states[s]).abs().max()) <= 5e-5 * max(1.0, float(states[s].abs().max())), s
+
+
+@pytest.mark.parametrize("pieces,seg", [(None, None), ([[300] + [1] * 60], None), ([[7] * 51 + [3]], None), (None, 64), ([[290, 70]], 32)])
+def test_a_state_keeps_what_it_was_given_hundreds_of_tokens_before(ops, pieces, seg):
     """Head 0 hardly decays (exp(A_log) = e^-9), head 1 forgets within a few tokens: the far token's B row meets the
     near token's C row in head 0 and stands out of everything in between; in head 1 nothing of it is left."""
     H, P_, N, G = 2, 16, 32, 1
     far, near = 11, 350
     for hd, kept in ((0, True), (1, False)):
         got, want, xbc, d_skip = scan_case(ops, torch.float32, H, P_, N, G, [360], pieces, seed=3, a_log=[-9.0, 1.5],
-                                           meet=(0, far, near, hd))
+                                           meet=(0, far, near, hd), seg_len=seg)
         assert float((got[0].double() - want[0]).abs().max()) <= 5e-5 * max(1.0, float(want[0].abs().max()))
         # what the far token alone would put out at the near one, undecayed: dt (B . C) x, dt = softplus(3 + bias) > 1
         y = want[0][near, hd * P_:(hd + 1) * P_] - d_skip[hd].double() * xbc[0][near, hd * P_:(hd + 1) * P_].double()
@@ -411,6 +441,29 @@ def test_mixers_whole_token_by_token_in_portions_and_in_batches(dtype, kind, kw)
     assert float((out[0] - plain(y)[29]).abs().max()) <= bound
     assert float((out[1:21] - want[50:70]).abs().max()) <= bound
     assert float((out[21:] - plain(u)).abs().max()) <= bound
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kw", [dict(), dict(W=128, H=2, P_=64, N=64, G=1, norm_groups=1, taps=4)])
+def test_state_mixer_with_portions_long_enough_for_segments(dtype, kw):
+    """A prompt of several segments whole; the same in two long portions and single tokens; a long portion of one request
+    beside a single token of another."""
+    h, plain = state_harness(dtype, **kw)
+    W = kw.get("W", 96)
+    T = 700
+    x = torch.randn(T, W, generator=gen(43)).to(dtype)
+    want = plain(x)
+    bound = tol(dtype, want, 5e-5, 3e-2)
+    assert float((h.mixer(x, [("whole", T)]) - want).abs().max()) <= bound
+    got = [h.mixer(x[:300], [("cut", 300)]), h.mixer(x[300:301], [("cut", 1)]), h.mixer(x[301:690], [("cut", 389)])]
+    got += [h.mixer(x[i:i + 1], [("cut", 1)]) for i in range(690, T)]
+    assert float((torch.cat(got) - want).abs().max()) <= bound
+    y = torch.randn(30, W, generator=gen(44)).to(dtype)
+    h.mixer(y[:29], [("b", 29)])
+    h.mixer(x[:130], [("a", 130)])
+    out = h.mixer(torch.cat([y[29:30], x[130:500]]), [("b", 1), ("a", 370)])
+    assert float((out[0] - plain(y)[29]).abs().max()) <= bound
+    assert float((out[1:] - want[130:500]).abs().max()) <= bound
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
