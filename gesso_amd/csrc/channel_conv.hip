@@ -7,8 +7,9 @@
 // K - 2 is the newest), zeros at a request's start.  act: 0 none, 1 silu.  The input may be a column range of wider
 // rows (ldx, the range starts at x).  Products and sums are float32, taps from j = 0 upward, whatever the cut.
 //
-//   channel_conv         one thread per (token, channel); a sequence that brings a single token also moves its history
-//                        on (nobody else reads it in this step)
+//   channel_conv         one thread per (token, channel), or per (token, eight channels) where widths and addresses
+//                        allow 16-byte accesses (the same sums in the same order); a sequence that brings a single
+//                        token also moves its history on (nobody else reads it in this step)
 //   channel_conv_state   one thread per (sequence, channel), for the sequences that bring more than one token: the new
 //                        history from the old one and the step's rows, read whole before anything is written
 #include "common.h"
@@ -49,6 +50,38 @@ __global__ void channel_conv_kernel(const TX* __restrict__ x, int ldx, const flo
   }
 }
 
+template <typename TX, typename TO>
+__global__ void channel_conv_vec_kernel(const TX* __restrict__ x, int ldx, const float* __restrict__ taps,
+                                        const float* __restrict__ bias, float* __restrict__ state,
+                                        const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
+                                        const int* __restrict__ slots, TO* __restrict__ out, int ldo, int T, int C, int K,
+                                        int act, int residual) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  const int C8 = C / 8;
+  if (i >= (long)T * C8) return;
+  const int t = (int)(i / C8), c = (int)(i % C8) * 8;
+  const int s = seq_of_token[t];
+  const int start = q_start[s], len = q_start[s + 1] - start;
+  float* hist = state + (size_t)slots[s] * (K - 1) * C + c;
+  float y[8], in[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y[e] = bias ? bias[c + e] : 0.f;
+  for (int j = 0; j < K; ++j) {
+    const int tt = t - (K - 1) + j;
+    if (tt >= start) load8f(x + (size_t)tt * ldx + c, in);
+    else load8f(hist + (size_t)(K - 1 + tt - start) * C, in);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = fmaf(taps[(size_t)(c + e) * K + j], in[e], y[e]);
+    if (len == 1 && j >= 1) store8f(hist + (size_t)(j - 1) * C, in);     // (row j - 1 was read one turn ago)
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    if (act == 1) y[e] = y[e] / (1.f + expf(-y[e]));
+    if (residual) y[e] += in[e];
+  }
+  store8f(out + (size_t)t * ldo + c, y);
+}
+
 template <typename TX>
 __global__ void channel_conv_state_kernel(const TX* __restrict__ x, int ldx, float* __restrict__ state,
                                           const int* __restrict__ q_start, const int* __restrict__ slots, int nseq, int C,
@@ -82,10 +115,18 @@ extern "C" int gs_channel_conv(const void* x, int x_dtype, int ldx, const float*
   GS_REQUIRE(ldx >= C && ldo >= C, "channel_conv: rows of %d and %d hold no %d channels", ldx, ldo, C);
   GS_REQUIRE(act == 0 || act == 1, "channel_conv: activation %d", act);
   if (T == 0) return 0;
-  const int blocks = gs_ceil_div((long)T * C, 256);
-#define GS_RUN(TX, TO)                                                                                              \
-  channel_conv_kernel<TX, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token, q_start, \
-                                                         slots, (TO*)out, ldo, T, C, K, act, residual)
+  const bool vec = C % 8 == 0 && ldx % 8 == 0 && ldo % 8 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)out | (uintptr_t)state) & 15) == 0;
+  const int blocks = gs_ceil_div((long)T * (vec ? C / 8 : C), 256);
+#define GS_RUN(TX, TO)                                                                                                    \
+  do {                                                                                                                    \
+    if (vec)                                                                                                              \
+      channel_conv_vec_kernel<TX, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token,     \
+                                                                 q_start, slots, (TO*)out, ldo, T, C, K, act, residual);  \
+    else                                                                                                                  \
+      channel_conv_kernel<TX, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token, q_start, \
+                                                             slots, (TO*)out, ldo, T, C, K, act, residual);               \
+  } while (0)
   if (x_dtype == GS_F32 && out_dtype == GS_F32)
     GS_RUN(float, float);
   else if (x_dtype == GS_BF16 && out_dtype == GS_BF16)

@@ -8,6 +8,7 @@
 //
 //   moe_router         one block per token: logits by wavefronts that walk a router row together (float32 sums in a
 //                      fixed order), softmax, choice and weights by the first wavefront
+//   moe_choose         softmax, choice and weights from logits that a product has left (float32), a wavefront a token
 //   clamped_glu        (rows, 2F) = gate | up  ->  (rows, F), the expert's activation; float32 arithmetic
 //   moe_routed_up      a[t, k, :] = activation of expert e_k's gate and up products    one block per (token, choice)
 //   moe_routed_down    y[t, :] = sum_k w_k (W_down[e_k] a[t, k, :] or x[t, :]) (+ shared[t, :])
@@ -23,37 +24,11 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
 
-template <typename T, typename TW>
-__global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ x, int ldx, const TW* __restrict__ wr,
-                                                         const float* __restrict__ correction, int top, int EA, int H,
-                                                         int* __restrict__ choice, float* __restrict__ weight) {
-  extern __shared__ float mr_sh[];           // H floats of the row, EA logits, EA choice scores, top chosen outputs
-  float* xs = mr_sh;
-  float* z = mr_sh + H;
-  float* cs = z + EA;
-  int* chosen = reinterpret_cast<int*>(cs + EA);
-  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) xs[j] = to_f32(x[(size_t)t * ldx + j]);
-  __syncthreads();
-  const bool vec = (H & 7) == 0 && aligned16(wr);
-  for (int e = wave; e < EA; e += nw) {
-    const TW* row = wr + (size_t)e * H;
-    float s = 0.f;
-    if (vec) {
-      for (int j = lane * 8; j < H; j += 512) {
-        float w8[8];
-        load8f(row + j, w8);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) s = fmaf(w8[i], xs[j + i], s);
-      }
-    } else {
-      for (int j = lane; j < H; j += 64) s = fmaf(to_f32(row[j]), xs[j], s);
-    }
-    s = wave_sum(s);
-    if (lane == 0) z[e] = s;
-  }
-  __syncthreads();
-  if (wave != 0) return;
+// One wavefront, from a token's logits in `z` (LDS, EA floats; `cs` as many, `chosen` top ints): softmax, the `top`
+// largest corrected scores (of equal ones the lowest index), the chosen ones' weights.
+__device__ __forceinline__ void route_from_logits(float* z, float* cs, int* chosen, const float* __restrict__ correction,
+                                                  int top, int EA, int lane, int t, int* __restrict__ choice,
+                                                  float* __restrict__ weight) {
   float m = -INFINITY;
   for (int e = lane; e < EA; e += 64) m = fmaxf(m, z[e]);
   m = wave_max(m);
@@ -98,6 +73,71 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ x
     choice[(size_t)t * top + k] = chosen[k];
     weight[(size_t)t * top + k] = z[chosen[k]] * inv;
   }
+}
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ x, int ldx, const TW* __restrict__ wr,
+                                                         const float* __restrict__ correction, int top, int EA, int H,
+                                                         int* __restrict__ choice, float* __restrict__ weight) {
+  extern __shared__ float mr_sh[];           // H floats of the row, EA logits, EA choice scores, top chosen outputs
+  float* xs = mr_sh;
+  float* z = mr_sh + H;
+  float* cs = z + EA;
+  int* chosen = reinterpret_cast<int*>(cs + EA);
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) xs[j] = to_f32(x[(size_t)t * ldx + j]);
+  __syncthreads();
+  const bool vec = (H & 7) == 0 && aligned16(wr);
+  // four rows of the router at a time per wavefront: their loads are in flight together, the token's features are read
+  // from LDS once for the four.  Each row's sum runs in the order it would run alone.
+  for (int e0 = wave * 4; e0 < EA; e0 += nw * 4) {
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    const TW* row[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) row[r] = wr + (size_t)(e0 + r < EA ? e0 + r : e0) * H;
+    if (vec) {
+      for (int j = lane * 8; j < H; j += 512) {
+        float w8[4][8];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) load8f(row[r] + j, w8[r]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xv = xs[j + i];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) s[r] = fmaf(w8[r][i], xv, s[r]);
+        }
+      }
+    } else {
+      for (int j = lane; j < H; j += 64) {
+        const float xv = xs[j];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[r] = fmaf(to_f32(row[r][j]), xv, s[r]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float all = wave_sum(s[r]);
+      if (lane == 0 && e0 + r < EA) z[e0 + r] = all;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight);
+}
+
+// The same from logits that a product has left: z (T, ldz) float32; one wavefront a token, four a block.
+__global__ __launch_bounds__(256) void moe_choose_kernel(const float* __restrict__ logits, int ldz,
+                                                         const float* __restrict__ correction, int top, int EA,
+                                                         int* __restrict__ choice, float* __restrict__ weight, int T) {
+  extern __shared__ float mc_sh[];           // per wavefront: EA logits, EA choice scores, top chosen outputs
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= T) return;
+  float* z = mc_sh + (size_t)wave * (2 * EA + top);
+  float* cs = z + EA;
+  int* chosen = reinterpret_cast<int*>(cs + EA);
+  for (int e = lane; e < EA; e += 64) z[e] = logits[(size_t)t * ldz + e];
+  route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight);
 }
 
 template <typename TI, typename TO>
@@ -239,6 +279,17 @@ extern "C" int gs_moe_router(const void* x, int dtype, int ldx, const void* wr, 
   else
     GS_REQUIRE(false, "moe_router: unsupported types %d %d", dtype, w_dtype);
   GS_LAUNCH_CHECK("moe_router");
+  return 0;
+}
+
+extern "C" int gs_moe_choose(const float* logits, int ldz, const float* correction, int top, int EA, int* choice,
+                             float* weight, int ntok, hipStream_t stream) {
+  GS_REQUIRE(ntok >= 0 && top > 0 && EA >= top && ldz >= EA, "moe_choose: bad sizes T=%d top=%d outputs=%d rows of %d", ntok, top, EA, ldz);
+  const size_t lds = 4 * (2 * (size_t)EA + (size_t)top) * sizeof(float);
+  GS_REQUIRE(lds <= 65536, "moe_choose: %d outputs are more than the kernel stages", EA);
+  if (ntok == 0) return 0;
+  moe_choose_kernel<<<gs_ceil_div(ntok, 4), 256, lds, stream>>>(logits, ldz, correction, top, EA, choice, weight, ntok);
+  GS_LAUNCH_CHECK("moe_choose");
   return 0;
 }
 

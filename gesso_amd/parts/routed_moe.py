@@ -17,6 +17,9 @@ from .base import MATRIX, VECTOR, Part, TensorSpec
 from .registry import register
 
 
+MANY_TOKENS = 256      # from this many tokens on the router's logits are a product of their own, then the choice
+
+
 class RoutedMoE(Part):
     graph_safe = True
     stage, out_stage = "moe_ffn", "ffn_down"
@@ -39,14 +42,20 @@ class RoutedMoE(Part):
 
     def bind(self, tensors):
         s, rt = self.spec, self.rt
-        self.router = tensors["router.weight"].contiguous()
+        router = self.router = tensors["router.weight"].contiguous()
+        # for steps of many tokens: the router's rows filled up to whole tiles of outputs with zeros; its logits are then
+        # a product like any other (float32 sums and results), of which the choice reads the first ``E + I`` columns.
+        # Steps of few tokens take one kernel for logits and choice
+        extra = -router.shape[0] % 16
+        padded = torch.cat([router, torch.zeros((extra, s.hidden), dtype=router.dtype, device=router.device)], 0)
+        self.w_router = rt.prepare(padded.contiguous())
         self.correction = tensors.get("router.correction")
         E = s.n_experts
         gus = [torch.cat([tensors[f"experts.{e}.gate.weight"], tensors[f"experts.{e}.up.weight"]], 0) for e in range(E)]
         downs = [tensors[f"experts.{e}.down.weight"] for e in range(E)]
         if len({w.dtype for w in gus + downs}) > 1:
             gus, downs = [w.float() for w in gus], [w.float() for w in downs]
-        dev, dt = self.router.device, (gus[0].dtype if E else self.router.dtype)
+        dev, dt = router.device, (gus[0].dtype if E else router.dtype)
         self.gate_up = torch.stack(gus, 0).contiguous() if E else torch.zeros((0, 2 * s.expert_ff, s.hidden), dtype=dt, device=dev)
         self.down = torch.stack(downs, 0).contiguous() if E else torch.zeros((0, s.hidden, s.expert_ff), dtype=dt, device=dev)
         self.w_sgu = self.w_sdown = None
@@ -61,7 +70,11 @@ class RoutedMoE(Part):
         s, rt, ops = self.spec, self.rt, self.rt.ops
         x = rt.dense(x)
         with rt.stage("ffn_router"):
-            choice, weight = ops.moe_router(x, self.router, self.correction, s.top)
+            if x.shape[0] >= MANY_TOKENS:
+                logits = rt.linear(x, self.w_router, out_dtype=torch.float32)
+                choice, weight = ops.moe_choose(logits, self.correction, s.top, s.n_experts + s.n_identity)
+            else:
+                choice, weight = ops.moe_router(x, self.router, self.correction, s.top)
         shared = None
         if self.w_sgu is not None:
             with rt.stage("ffn_shared"):

@@ -84,7 +84,7 @@ def conv_case(ops, dtype, C, K, lens, pieces, act=None, residual=False, bias=Tru
     """Sequences of ``lens`` tokens, each fed in the pieces ``pieces[s]`` (steps hold piece i of every sequence that has
     one), histories in shuffled slots.  Returns the kernel's rows and the plain convolution's, per sequence."""
     g = gen(seed)
-    junk = 3
+    junk = 8 if C % 16 == 0 else 3          # (rows whose stride and start allow 16-byte accesses, and rows that do not)
     xs = [(torch.randn(n, C + junk, generator=g) * 1.5).to(dtype) for n in lens]
     taps = torch.randn(C, K, generator=g) * 0.5
     b = torch.randn(C, generator=g) if bias else None
@@ -122,7 +122,7 @@ def conv_case(ops, dtype, C, K, lens, pieces, act=None, residual=False, bias=Tru
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,K", [(40, 4), (33, 3), (130, 2), (17, 5), (24, 1), (520, 4)])
+@pytest.mark.parametrize("C,K", [(40, 4), (33, 3), (130, 2), (17, 5), (24, 1), (520, 4), (48, 4), (64, 1), (528, 3), (16, 5)])
 def test_convolution_over_time_in_pieces_with_a_history_per_request(ops, dtype, C, K):
     lens = [1, 23, 2, 12, 9]
     pieces = [[1], [5, 1, 1, 2, 7, 3, 1, 3], [1, 1], [12], [2, 2, 1, 1, 3]]
@@ -284,6 +284,12 @@ def test_router_chooses_by_corrected_scores_and_weighs_by_plain_ones(ops, dtype,
     assert torch.equal(choice.cpu().long()[clear], want_c[clear])
     assert float((weight.cpu().double()[clear] - want_w[clear]).abs().max()) <= 2e-5
     assert float((weight.sum(1) - 1).abs().max()) <= 1e-5
+    # the same from logits that a product has left, in rows wider than the router's outputs
+    logits = torch.full((50, EA + 5), 1e9)
+    logits[:, :EA] = P.linear(x.double(), router.double()).float()
+    c2, w2 = ops.moe_choose(logits.to(DEV), correction.to(DEV), top, EA)
+    assert torch.equal(c2.cpu().long()[clear], want_c[clear])
+    assert float((w2.cpu().double()[clear] - want_w[clear]).abs().max()) <= 2e-5
     # equal scores (a router of zeros): the lowest indices, equal weights
     zc, zw = ops.moe_router(x.to(DEV), torch.zeros_like(router).to(DEV), None, top)
     assert torch.equal(zc.cpu(), torch.arange(top, dtype=torch.int32).expand(50, top))
