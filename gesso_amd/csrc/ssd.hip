@@ -159,7 +159,8 @@ __global__ void ssd_combine_kernel(const float* __restrict__ state, const int* _
   }
 }
 
-extern "C" int gs_ssd_max_state() { return 512; }
+// The most state rows a head of P value columns may have: 64 a thread, eight row groups for narrow heads, else four.
+extern "C" int gs_ssd_max_state(int P) { return 64 * (P <= 32 ? 8 : 4); }
 
 template <typename TD, int PC, int MODE>
 static int ssd_launch(int nk, dim3 grid, hipStream_t stream, const float* xbc, int ldx, int ob, int oc, const TD* drows,

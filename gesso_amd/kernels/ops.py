@@ -1376,8 +1376,9 @@ def channel_conv(x, taps, bias, state, seq_of_token, q_start, slots, nseq: int, 
 
 # ---------------------------------------------------------------------- a state-space recurrence
 
-def ssd_max_state() -> int:
-    return int(lib().gs_ssd_max_state())
+def ssd_max_state(P: int) -> int:
+    """The most state rows :func:`ssd_scan` holds for heads of ``P`` value columns."""
+    return int(lib().gs_ssd_max_state(int(P)))
 
 
 def ssd_scan(xbc, rows, odt: int, dt_bias, a_log, d_skip, state, q_start, slots, nseq: int, H: int, P: int, N: int,

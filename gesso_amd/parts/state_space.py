@@ -36,8 +36,9 @@ class StateSpace(Part):
             raise ValueError(f"{spec.n_heads} heads do not share {spec.groups} groups evenly")
         if (spec.n_heads * spec.head_dim) % spec.norm_groups:
             raise ValueError(f"{spec.norm_groups} norm parts do not divide {spec.n_heads * spec.head_dim} features")
-        if spec.state > rt.ops.ssd_max_state():
-            raise ValueError(f"a state of {spec.state} rows: the state kernel holds up to {rt.ops.ssd_max_state()}")
+        if spec.state > rt.ops.ssd_max_state(spec.head_dim):
+            raise ValueError(f"a state of {spec.state} rows: the state kernel holds up to "
+                             f"{rt.ops.ssd_max_state(spec.head_dim)} for heads of {spec.head_dim}")
 
     @staticmethod
     def sizes(spec):
