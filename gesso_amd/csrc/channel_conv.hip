@@ -50,11 +50,13 @@ __global__ void channel_conv_kernel(const TX* __restrict__ x, int ldx, const flo
   }
 }
 
-template <typename TX, typename TO>
+// Eight channels a thread; K is the number of taps, known at compile time: the thread's 8 K taps lie side by side in
+// memory and are read as 16-byte pieces into registers.
+template <typename TX, typename TO, int K>
 __global__ void channel_conv_vec_kernel(const TX* __restrict__ x, int ldx, const float* __restrict__ taps,
                                         const float* __restrict__ bias, float* __restrict__ state,
                                         const int* __restrict__ seq_of_token, const int* __restrict__ q_start,
-                                        const int* __restrict__ slots, TO* __restrict__ out, int ldo, int T, int C, int K,
+                                        const int* __restrict__ slots, TO* __restrict__ out, int ldo, int T, int C,
                                         int act, int residual) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   const int C8 = C / 8;
@@ -63,21 +65,37 @@ __global__ void channel_conv_vec_kernel(const TX* __restrict__ x, int ldx, const
   const int s = seq_of_token[t];
   const int start = q_start[s], len = q_start[s + 1] - start;
   float* hist = state + (size_t)slots[s] * (K - 1) * C + c;
-  float y[8], in[8];
+  float w[8 * K];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) y[e] = bias ? bias[c + e] : 0.f;
+  for (int q = 0; q < 2 * K; ++q) {
+    const float4 v = reinterpret_cast<const float4*>(taps + (size_t)c * K)[q];
+    w[4 * q] = v.x; w[4 * q + 1] = v.y; w[4 * q + 2] = v.z; w[4 * q + 3] = v.w;
+  }
+  float y[8], in[K][8];
+  if (bias) load8f(bias + c, y);
+  else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = 0.f;
+  }
+#pragma unroll
   for (int j = 0; j < K; ++j) {
     const int tt = t - (K - 1) + j;
-    if (tt >= start) load8f(x + (size_t)tt * ldx + c, in);
-    else load8f(hist + (size_t)(K - 1 + tt - start) * C, in);
+    if (tt >= start) load8f(x + (size_t)tt * ldx + c, in[j]);
+    else load8f(hist + (size_t)(K - 1 + tt - start) * C, in[j]);
+  }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = fmaf(taps[(size_t)(c + e) * K + j], in[e], y[e]);
-    if (len == 1 && j >= 1) store8f(hist + (size_t)(j - 1) * C, in);     // (row j - 1 was read one turn ago)
+  for (int j = 0; j < K; ++j) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = fmaf(w[e * K + j], in[j][e], y[e]);
+  }
+  if (len == 1) {
+#pragma unroll
+    for (int j = 1; j < K; ++j) store8f(hist + (size_t)(j - 1) * C, in[j]);     // (every row was read above)
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     if (act == 1) y[e] = y[e] / (1.f + expf(-y[e]));
-    if (residual) y[e] += in[e];
+    if (residual) y[e] += in[K - 1][e];
   }
   store8f(out + (size_t)t * ldo + c, y);
 }
@@ -115,14 +133,19 @@ extern "C" int gs_channel_conv(const void* x, int x_dtype, int ldx, const float*
   GS_REQUIRE(ldx >= C && ldo >= C, "channel_conv: rows of %d and %d hold no %d channels", ldx, ldo, C);
   GS_REQUIRE(act == 0 || act == 1, "channel_conv: activation %d", act);
   if (T == 0) return 0;
-  const bool vec = C % 8 == 0 && ldx % 8 == 0 && ldo % 8 == 0 &&
-                   (((uintptr_t)x | (uintptr_t)out | (uintptr_t)state) & 15) == 0;
+  const bool vec = C % 8 == 0 && ldx % 8 == 0 && ldo % 8 == 0 && K <= 5 &&
+                   (((uintptr_t)x | (uintptr_t)out | (uintptr_t)state | (uintptr_t)taps | (uintptr_t)bias) & 15) == 0;
   const int blocks = gs_ceil_div((long)T * (vec ? C / 8 : C), 256);
+#define GS_VEC(TX, TO, KK)                                                                                              \
+  channel_conv_vec_kernel<TX, TO, KK><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token,   \
+                                                                 q_start, slots, (TO*)out, ldo, T, C, act, residual)
 #define GS_RUN(TX, TO)                                                                                                    \
   do {                                                                                                                    \
-    if (vec)                                                                                                              \
-      channel_conv_vec_kernel<TX, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token,     \
-                                                                 q_start, slots, (TO*)out, ldo, T, C, K, act, residual);  \
+    if (vec && K == 1) GS_VEC(TX, TO, 1);                                                                                 \
+    else if (vec && K == 2) GS_VEC(TX, TO, 2);                                                                            \
+    else if (vec && K == 3) GS_VEC(TX, TO, 3);                                                                            \
+    else if (vec && K == 4) GS_VEC(TX, TO, 4);                                                                            \
+    else if (vec) GS_VEC(TX, TO, 5);                                                                                      \
     else                                                                                                                  \
       channel_conv_kernel<TX, TO><<<blocks, 256, 0, stream>>>((const TX*)x, ldx, taps, bias, state, seq_of_token, q_start, \
                                                              slots, (TO*)out, ldo, T, C, K, act, residual);               \
@@ -136,6 +159,7 @@ extern "C" int gs_channel_conv(const void* x, int x_dtype, int ldx, const float*
   else
     GS_REQUIRE(false, "channel_conv: unknown dtypes %d %d", x_dtype, out_dtype);
 #undef GS_RUN
+#undef GS_VEC
   GS_LAUNCH_CHECK("channel_conv");
   if (!all_single && K > 1) {
     const int sb = gs_ceil_div((long)nseq * C, 256);

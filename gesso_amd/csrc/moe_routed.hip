@@ -96,15 +96,23 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ x
 #pragma unroll
     for (int r = 0; r < 4; ++r) row[r] = wr + (size_t)(e0 + r < EA ? e0 + r : e0) * H;
     if (vec) {
-      for (int j = lane * 8; j < H; j += 512) {
-        float w8[4][8];
+      // two steps of 512 columns at a time: eight loads in flight a lane
+      for (int j = lane * 8; j < H; j += 1024) {
+        const bool two = j + 512 < H;
+        float w8[2][4][8];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) load8f(row[r] + j, w8[r]);
+        for (int r = 0; r < 4; ++r) load8f(row[r] + j, w8[0][r]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float xv = xs[j + i];
+        for (int r = 0; r < 4; ++r) load8f(row[r] + (two ? j + 512 : j), w8[1][r]);
 #pragma unroll
-          for (int r = 0; r < 4; ++r) s[r] = fmaf(w8[r][i], xv, s[r]);
+        for (int u = 0; u < 2; ++u) {
+          if (u == 1 && !two) break;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const float xv = xs[j + 512 * u + i];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[r] = fmaf(w8[u][r][i], xv, s[r]);
+          }
         }
       }
     } else {

@@ -138,17 +138,19 @@ def test_convolution_over_time_in_pieces_with_a_history_per_request(ops, dtype, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,groups", [(64, 2), (96, 3), (90, 1), (256, 4), (60, 6)])
+@pytest.mark.parametrize("H,groups", [(64, 2), (96, 3), (90, 1), (256, 4), (60, 6), (2048, 1), (4096, 8), (48, 3), (64, 16)])
 def test_gate_then_norm_in_parts(ops, dtype, H, groups):
     y = torch.randn(9, H, generator=gen(4)) * 2
     y[:, :H // groups] *= 30
-    wide = torch.randn(9, H + 11, generator=gen(5)).to(dtype)                 # the gate: a column range of wider rows
+    # the gate: a column range of wider rows (with and without a start and a stride that allow 16-byte accesses)
+    at, extra = (8, 16) if H % 16 == 0 else (4, 11)
+    wide = torch.randn(9, H + extra, generator=gen(5)).to(dtype)
     w = 1 + 0.3 * torch.randn(H, generator=gen(6))
-    got = ops.gated_group_norm(y.to(DEV), wide.to(DEV)[:, 4:4 + H], w.to(DEV), 1e-6, groups, dtype).double().cpu()
-    want = P.group_norm(y.double() * P.silu(wide[:, 4:4 + H].double()), w.double(), 1e-6, groups)
+    got = ops.gated_group_norm(y.to(DEV), wide.to(DEV)[:, at:at + H], w.to(DEV), 1e-6, groups, dtype).double().cpu()
+    want = P.group_norm(y.double() * P.silu(wide[:, at:at + H].double()), w.double(), 1e-6, groups)
     assert float((got - want).abs().max()) <= tol(dtype, want)
     # the other order (norm, then gate) is another function: the inputs tell them apart
-    other = P.group_norm(y.double(), w.double(), 1e-6, groups) * P.silu(wide[:, 4:4 + H].double())
+    other = P.group_norm(y.double(), w.double(), 1e-6, groups) * P.silu(wide[:, at:at + H].double())
     assert float((other - want).abs().max()) > 10 * tol(dtype, want)
 
 
@@ -404,6 +406,7 @@ def harness(kind, dtype, **kw):
 CASES = [("state", dict()), ("state", dict(W=64, H=3, P_=24, N=16, G=1, norm_groups=3, taps=3)),
          ("state", dict(W=64, H=6, P_=8, N=12, G=3, norm_groups=6, taps=2)), ("state", dict(W=128, H=2, P_=64, N=64, G=1, norm_groups=1, taps=4)),
          ("state", dict(W=100, H=5, P_=10, N=7, G=5, norm_groups=2, taps=1)), ("state", dict(W=128, H=2, P_=128, N=128, G=2, norm_groups=1, taps=5)),
+         ("state", dict(W=128, H=8, P_=32, N=48, G=2, norm_groups=2, taps=4)),
          ("latent", dict()), ("latent", dict(W=64, H=2, n=8, r=16, dv=24, qr=24, c=32)),
          ("latent", dict(W=64, H=1, n=24, r=8, dv=16, qr=16, c=36, base=100.0)), ("latent", dict(W=100, H=5, n=0, r=6, dv=14, qr=18, c=22, base=3e4)),
          ("latent", dict(W=100, H=2, n=18, r=2, dv=6, qr=10, c=30)), ("latent", dict(W=128, H=4, n=64, r=64, dv=64, qr=64, c=128, base=5e5, page_size=16)),
