@@ -24,6 +24,21 @@ __device__ __forceinline__ float clamped_glu(float g, float u, float limit, floa
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
 
+// A row of H values into LDS as float32, by the whole block: 16-byte reads where the row allows them.
+template <typename T>
+__device__ __forceinline__ void stage_row(float* xs, const T* __restrict__ row, int H) {
+  if ((H & 7) == 0 && aligned16(row)) {
+    for (int j = threadIdx.x * 8; j < H; j += blockDim.x * 8) {
+      float v[8];
+      load8f(row + j, v);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xs[j + e] = v[e];
+    }
+  } else {
+    for (int j = threadIdx.x; j < H; j += blockDim.x) xs[j] = to_f32(row[j]);
+  }
+}
+
 // One wavefront, from a token's logits in `z` (LDS, EA floats; `cs` as many, `chosen` top ints): softmax, the `top`
 // largest corrected scores (of equal ones the lowest index), the chosen ones' weights.
 __device__ __forceinline__ void route_from_logits(float* z, float* cs, int* chosen, const float* __restrict__ correction,
@@ -85,7 +100,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const T* __restrict__ x
   float* cs = z + EA;
   int* chosen = reinterpret_cast<int*>(cs + EA);
   const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) xs[j] = to_f32(x[(size_t)t * ldx + j]);
+  stage_row(xs, x + (size_t)t * ldx, H);
   __syncthreads();
   const bool vec = (H & 7) == 0 && aligned16(wr);
   // four rows of the router at a time per wavefront: their loads are in flight together, the token's features are read
@@ -167,7 +182,7 @@ __global__ void moe_routed_up_kernel(const T* __restrict__ x, int ldx, const int
   const int e = choice[(size_t)t * top + k];
   if (e >= E) return;                // an identity expert has no inner values
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-  for (int j = threadIdx.x; j < H; j += blockDim.x) xs[j] = to_f32(x[(size_t)t * ldx + j]);
+  stage_row(xs, x + (size_t)t * ldx, H);
   __syncthreads();
   const TW* w = gate_up + (size_t)e * 2 * F * H;
   T* dst = a + ((size_t)t * top + k) * F;

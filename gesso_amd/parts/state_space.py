@@ -23,7 +23,7 @@ from .base import MATRIX, VECTOR, Part, SlotState, TensorSpec
 from .registry import register
 
 
-SEGMENT = 128      # tokens a segment: long portions are walked in segments of this many, side by side
+SEGMENT = 128      # tokens a segment: long portions are walked in segments of this many (or half), side by side
 
 
 class StateSpace(Part):
@@ -81,7 +81,11 @@ class StateSpace(Part):
                                    activation="silu")
         with rt.stage("state_scan"):
             # a step that brings a long portion: its segments side by side instead of one walk a sequence and head
-            segments = ctx.state_segments(SEGMENT) if ctx.max_q_len >= 2 * SEGMENT else None
+            segments = None
+            if ctx.max_q_len >= 2 * SEGMENT:
+                # shorter segments while the longer ones would leave compute units with fewer than four blocks
+                blocks = (ctx.T // SEGMENT) * H * -(-P // 64)
+                segments = ctx.state_segments(SEGMENT if blocks >= 4 * rt.compute_units else SEGMENT // 2)
             y = ops.ssd_scan(xbc, rows, inner + chan, self.dt_bias, self.a_log, self.d_skip, cache.state["state"],
                              ctx.q_start, ctx.slots, ctx.nseq, H, P, N, G, segments=segments)
         with rt.stage("state_norm"):
