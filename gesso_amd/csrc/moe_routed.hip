@@ -6,9 +6,8 @@
 //     g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = W_down (g sigmoid(alpha g) (u + 1)).
 //   Expert weights lie stacked: gate_up (E, 2F, H) (a gate's rows, then the up rows), down (E, H, F).
 //
-//   moe_router         one block per token: logits by wavefronts that walk a router row together (float32 sums in a
-//                      fixed order), softmax, choice and weights by the first wavefront
-//   moe_choose         softmax, choice and weights from logits that a product has left (float32), a wavefront a token
+//   moe_router         one block per token, a wavefront for every four router rows: logits by wavefronts that walk
+//                      their rows together (float32 sums in a fixed order), softmax, choice and weights by the first
 //   clamped_glu        (rows, 2F) = gate | up  ->  (rows, F), the expert's activation; float32 arithmetic
 //   moe_routed_up      a[t, k, :] = activation of expert e_k's gate and up products    one block per (token, choice)
 //   moe_routed_down    y[t, :] = sum_k w_k (W_down[e_k] a[t, k, :] or x[t, :]) (+ shared[t, :])
@@ -145,21 +144,6 @@ __global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ 
   }
   __syncthreads();
   if (wave != 0) return;
-  route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight);
-}
-
-// The same from logits that a product has left: z (T, ldz) float32; one wavefront a token, four a block.
-__global__ __launch_bounds__(256) void moe_choose_kernel(const float* __restrict__ logits, int ldz,
-                                                         const float* __restrict__ correction, int top, int EA,
-                                                         int* __restrict__ choice, float* __restrict__ weight, int T) {
-  extern __shared__ float mc_sh[];           // per wavefront: EA logits, EA choice scores, top chosen outputs
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = blockIdx.x * 4 + wave;
-  if (t >= T) return;
-  float* z = mc_sh + (size_t)wave * (2 * EA + top);
-  float* cs = z + EA;
-  int* chosen = reinterpret_cast<int*>(cs + EA);
-  for (int e = lane; e < EA; e += 64) z[e] = logits[(size_t)t * ldz + e];
   route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight);
 }
 
@@ -325,17 +309,6 @@ extern "C" int gs_moe_router(const void* x, int dtype, int ldx, const void* wr, 
   else
     GS_REQUIRE(false, "moe_router: unsupported types %d %d", dtype, w_dtype);
   GS_LAUNCH_CHECK("moe_router");
-  return 0;
-}
-
-extern "C" int gs_moe_choose(const float* logits, int ldz, const float* correction, int top, int EA, int* choice,
-                             float* weight, int ntok, hipStream_t stream) {
-  GS_REQUIRE(ntok >= 0 && top > 0 && EA >= top && ldz >= EA, "moe_choose: bad sizes T=%d top=%d outputs=%d rows of %d", ntok, top, EA, ldz);
-  const size_t lds = 4 * (2 * (size_t)EA + (size_t)top) * sizeof(float);
-  GS_REQUIRE(lds <= 65536, "moe_choose: %d outputs are more than the kernel stages", EA);
-  if (ntok == 0) return 0;
-  moe_choose_kernel<<<gs_ceil_div(ntok, 4), 256, lds, stream>>>(logits, ldz, correction, top, EA, choice, weight, ntok);
-  GS_LAUNCH_CHECK("moe_choose");
   return 0;
 }
 

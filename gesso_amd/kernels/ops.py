@@ -1433,21 +1433,6 @@ def moe_router(x, router, correction, top: int):
     return choice, weight
 
 
-def moe_choose(logits, correction, top: int, EA: int):
-    """:func:`moe_router` from logits that a product has left: ``logits (T, >= EA)`` float32, of which the first ``EA``
-    columns are the router's outputs.  Returns ``(choice int32 (T, top), weight float32 (T, top))``."""
-    _dev(logits, correction)
-    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1 and logits.shape[1] >= EA >= top >= 1,
-          "moe_choose: logits are float32 (T, at least the router's outputs), top within the outputs")
-    _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (EA,)), "moe_choose: the correction must be float32 (outputs,)")
-    T = logits.shape[0]
-    choice = torch.empty((T, top), dtype=torch.int32, device=logits.device)
-    weight = torch.empty((T, top), dtype=torch.float32, device=logits.device)
-    _check(lib().gs_moe_choose(_p(logits), logits.stride(0) if T > 1 else logits.shape[1], _p(correction), top, EA,
-                               _p(choice), _p(weight), T, _stream()))
-    return choice, weight
-
-
 def clamped_glu(gu, limit: float, alpha: float, out_dtype) -> torch.Tensor:
     """``gu (rows, 2F)`` = gate | up  ->  ``g sigmoid(alpha g) (u + 1)`` with ``g = min(gate, limit)``,
     ``u = clamp(up, -limit, limit)``: ``(rows, F)`` in ``out_dtype``, float32 arithmetic."""

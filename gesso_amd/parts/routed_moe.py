@@ -17,9 +17,6 @@ from .base import MATRIX, VECTOR, Part, TensorSpec
 from .registry import register
 
 
-MANY_TOKENS = 256      # from this many tokens on the router's logits are a product of their own, then the choice
-
-
 class RoutedMoE(Part):
     graph_safe = True
     stage, out_stage = "moe_ffn", "ffn_down"
@@ -43,12 +40,6 @@ class RoutedMoE(Part):
     def bind(self, tensors):
         s, rt = self.spec, self.rt
         router = self.router = tensors["router.weight"].contiguous()
-        # for steps of many tokens: the router's rows filled up to whole tiles of outputs with zeros; its logits are then
-        # a product like any other (float32 sums and results), of which the choice reads the first ``E + I`` columns.
-        # Steps of few tokens take one kernel for logits and choice
-        extra = -router.shape[0] % 16
-        padded = torch.cat([router, torch.zeros((extra, s.hidden), dtype=router.dtype, device=router.device)], 0)
-        self.w_router = rt.prepare(padded.contiguous())
         self.correction = tensors.get("router.correction")
         E = s.n_experts
         gus = [torch.cat([tensors[f"experts.{e}.gate.weight"], tensors[f"experts.{e}.up.weight"]], 0) for e in range(E)]
@@ -70,11 +61,7 @@ class RoutedMoE(Part):
         s, rt, ops = self.spec, self.rt, self.rt.ops
         x = rt.dense(x)
         with rt.stage("ffn_router"):
-            if x.shape[0] >= MANY_TOKENS:
-                logits = rt.linear(x, self.w_router, out_dtype=torch.float32)
-                choice, weight = ops.moe_choose(logits, self.correction, s.top, s.n_experts + s.n_identity)
-            else:
-                choice, weight = ops.moe_router(x, self.router, self.correction, s.top)
+            choice, weight = ops.moe_router(x, self.router, self.correction, s.top)
         shared = None
         if self.w_sgu is not None:
             with rt.stage("ffn_shared"):

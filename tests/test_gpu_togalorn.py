@@ -286,12 +286,6 @@ def test_router_chooses_by_corrected_scores_and_weighs_by_plain_ones(ops, dtype,
     assert torch.equal(choice.cpu().long()[clear], want_c[clear])
     assert float((weight.cpu().double()[clear] - want_w[clear]).abs().max()) <= 2e-5
     assert float((weight.sum(1) - 1).abs().max()) <= 1e-5
-    # the same from logits that a product has left, in rows wider than the router's outputs
-    logits = torch.full((50, EA + 5), 1e9)
-    logits[:, :EA] = P.linear(x.double(), router.double()).float()
-    c2, w2 = ops.moe_choose(logits.to(DEV), correction.to(DEV), top, EA)
-    assert torch.equal(c2.cpu().long()[clear], want_c[clear])
-    assert float((w2.cpu().double()[clear] - want_w[clear]).abs().max()) <= 2e-5
     # equal scores (a router of zeros): the lowest indices, equal weights
     zc, zw = ops.moe_router(x.to(DEV), torch.zeros_like(router).to(DEV), None, top)
     assert torch.equal(zc.cpu(), torch.arange(top, dtype=torch.int32).expand(50, top))
