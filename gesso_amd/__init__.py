@@ -9,6 +9,7 @@ from .models import lfm2 as _lfm2  # noqa: F401  registers the architecture
 from .models import makuzen as _makuzen  # noqa: F401  registers the architecture
 from .models import fazezen as _fazezen  # noqa: F401  registers the architecture
 from .models import togalorn as _togalorn  # noqa: F401  registers the architecture
+from .models import kuditar as _kuditar  # noqa: F401  registers the architecture
 from .errors import (ConfigError, GessoError, InvalidPlan, KernelError, NumericalInstability, OutOfPages,
                      OutOfSlots, ResourceLimit, StepFailed, WeightError)
 

@@ -203,9 +203,10 @@ class CacheManager:
             first_needed = group.need.first_needed(rc.length)     # oldest key the next query reads
             passed = max(0, first_needed) // self.page_size
             table = rc.tables[g]
-            gone = [table[b] for b in range(min(passed, len(table))) if table[b] != RELEASED]
+            kept = group.need.pages_kept(self.page_size)        # a sequence's first pages that a window never passes
+            gone = [table[b] for b in range(kept, min(passed, len(table))) if table[b] != RELEASED]
             if gone:
-                for b in range(min(passed, len(table))):
+                for b in range(kept, min(passed, len(table))):
                     table[b] = RELEASED
                 self.pools[g].give_back(gone)
                 if self.track_released:

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass
-from typing import Callable, Dict
+from typing import Callable, Dict, Optional
 
 from ..errors import ConfigError
 from .jsonio import load_strict
@@ -23,15 +23,18 @@ class Architecture:
     parse: Callable[[dict], object]          # config.json keys -> typed configuration
     to_spec: Callable[[object], ModelSpec]   # typed configuration -> model as data
     to_json: Callable[[object], dict]        # typed configuration -> config.json keys
+    # sizes that a design leaves to its tensors' shapes: ``complete(raw, shape_of) -> raw`` fills them into the file's
+    # keys before they are parsed; ``shape_of(tensor name)`` gives a stored tensor's shape, or None (None: no such sizes)
+    complete: Optional[Callable[[dict, Callable], dict]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, parse, to_spec, to_json) -> None:
+def register_architecture(name: str, parse, to_spec, to_json, complete=None) -> None:
     if name in _ARCHITECTURES:
         raise ConfigError(f"architecture {name!r} is already registered")
-    _ARCHITECTURES[name] = Architecture(name, parse, to_spec, to_json)
+    _ARCHITECTURES[name] = Architecture(name, parse, to_spec, to_json, complete)
 
 
 def unregister_architecture(name: str) -> None:
@@ -59,4 +62,24 @@ def load_config(model_dir: str):
     """``(architecture entry, typed configuration)`` of a model folder."""
     raw = load_strict(os.path.join(model_dir, "config.json"))
     arch = architecture_of(raw)
+    if arch.complete is not None:
+        raw = arch.complete(raw, _shapes_of(model_dir))
     return arch, arch.parse(raw)
+
+
+def _shapes_of(model_dir: str):
+    """``tensor name -> shape or None`` over the folder's weight files; only their headers are read, and only when
+    somebody asks."""
+    held = {}
+
+    def shape_of(name: str):
+        if not held:
+            from ..weights.safetensors_io import open_model_files
+            held["shapes"] = {}
+            for f in open_model_files(model_dir):
+                for n in f.names():
+                    held["shapes"][n] = tuple(f.shape(n))
+                f.close()
+        return held["shapes"].get(name)
+
+    return shape_of

@@ -31,6 +31,17 @@ class RMSNormSpec:
 
 
 @dataclass(frozen=True)
+class LayerNormSpec:
+    """``(x - mean(x)) / sqrt(var(x) + eps) * w + b``, the variance the mean of the squared deviations; ``bias``: whether
+    there is a ``b``."""
+
+    size: int
+    eps: float
+    bias: bool = True
+    kind: str = "layernorm"
+
+
+@dataclass(frozen=True)
 class GroupRMSNormSpec:
     """RMS norm in parts: the row is cut into ``groups`` equal consecutive parts, each is divided by its own
     ``sqrt(mean(part^2) + eps)``, and the whole is multiplied by the weight."""
@@ -52,6 +63,7 @@ class RopeSpec:
     max_position: int
     layout: str = "half"
     kind: str = "rope"
+    frequency_divisor: float = 1.0     # every pair's frequency is divided by this (positions stretched evenly)
 
 
 @dataclass(frozen=True)
@@ -121,6 +133,16 @@ class AttentionSpec:
     sink: bool = False                 # the softmax's denominator has one more term, exp(0), which has no value
     value_position: Any = None         # a position-encoding spec: values are cached turned by their own position, a
                                        # head's weighted sum is turned back by the query's
+    qk_norm_weight: bool = True        # False: the head norm of q and k has no weight (it may then stand after the
+                                       # turn as well as before it: a turn keeps a head's sum of squares)
+    out_bias: Optional[bool] = None    # whether the output projection has a bias (None: as ``bias``)
+    softcap: Optional[float] = None    # scores become softcap * tanh(score / softcap)
+    keep_first: int = 0                # with a window: the first positions of a sequence that stay visible beyond it
+    head_sinks: bool = False           # the softmax's denominator has one more term exp(s_h), s_h a stored number a head
+    out_gate: Optional[str] = None     # "sigmoid": the heads side by side are multiplied by sigmoid(W_g x) before the
+                                       # output projection
+    value_mix: bool = False            # the mixers that say so share values: the first of them to run in a step keeps
+                                       # its values v_first, each later one caches (1 - m) v + m v_first, m a stored number
 
 
 @dataclass(frozen=True)
@@ -176,15 +198,55 @@ class LinearAttentionSpec:
 
 
 @dataclass(frozen=True)
+class GatedDeltaSpec:
+    """The gated delta rule.  ``q, k`` (``qk_heads`` heads of ``key_dim``) and ``v`` (``n_heads`` of ``value_dim``) are
+    products of the input that pass a causal convolution over time per channel (``conv_taps`` taps, no bias) and silu;
+    q and k become unit vectors per head (``x / sqrt(sum(x^2) + unit_eps)``), q also times ``key_dim^-0.5``; head ``h``
+    uses q/k head ``h // (n_heads / qk_heads)``.  ``beta = sigmoid(W_b x)`` and
+    ``g = exp(-exp(A_log) softplus(W_a x + dt_bias))`` per head; ``S <- g S; u = beta (v - S^T k); S <- S + k u^T;
+    o = S^T q``; each head's ``o`` is RMS-normed with a weight of ``value_dim``, times ``silu(W_g x)``, then projected."""
+
+    hidden: int
+    n_heads: int
+    qk_heads: int
+    key_dim: int
+    value_dim: int
+    conv_taps: int
+    eps: float
+    unit_eps: float = 1e-6
+    kind: str = "gated_delta"
+
+
+@dataclass(frozen=True)
+class GatedLinearSpec:
+    """Linear attention with a decay per key channel: ``alpha = sigmoid(W_up (W_down x) + b)^(1/tau)`` (the decay's
+    product goes through ``decay_rank`` features), ``S_t = diag(alpha_t) S_(t-1) + k_t v_t^T``,
+    ``o_t = S_t^T (q_t key_dim^-0.5)``; each head's ``o`` is RMS-normed with a weight of ``value_dim``, times
+    ``silu(W_g x)``, then projected."""
+
+    hidden: int
+    n_heads: int
+    key_dim: int
+    value_dim: int
+    decay_rank: int
+    tau: float
+    eps: float
+    kind: str = "gated_linear"
+
+
+@dataclass(frozen=True)
 class MixerPairSpec:
     """Two mixers side by side that read the same input: ``left_scale * left(x) + right_scale * right(x)``.  Each keeps
-    its own cache."""
+    its own cache.  ``branch_norm_eps``: each side's output is first RMS-normed over the model width with a weight of
+    its own (``left_norm.weight``, ``right_norm.weight``); None: the outputs as they are."""
 
     left: Any
     right: Any
     left_scale: float = 1.0
     right_scale: float = 1.0
     kind: str = "mixer_pair"
+    branch_norm_eps: Optional[float] = None
+    hidden: Optional[int] = None       # the model width (the branch norms' size)
 
 
 @dataclass(frozen=True)
@@ -212,6 +274,18 @@ class GatedMLPSpec:
     activation: str = "gelu_tanh"
     bias: bool = True
     kind: str = "gated_mlp"
+
+
+@dataclass(frozen=True)
+class ClampedGLUSpec:
+    """``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate x, limit)``, ``u = clamp(W_up x, -limit, limit)``;
+    no biases."""
+
+    hidden: int
+    intermediate: int
+    limit: float
+    alpha: float = 1.702
+    kind: str = "clamped_glu"
 
 
 @dataclass(frozen=True)
@@ -259,7 +333,8 @@ class RoutedMoESpec:
     chosen scores' sum (+ 1e-20).  The last ``n_identity`` outputs name no weights: such an expert gives back its input.
     An expert is ``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate x, limit)``,
     ``u = clamp(W_up x, -limit, limit)``.  ``shared_ff``: a further expert of that width and ``shared_limit`` runs for every
-    token and is added (None: none)."""
+    token and is added (None: none).  ``score = "sigmoid"``: the scores are each output's sigmoid instead of their
+    softmax; ``renormalize = False``: the weights are the chosen scores as they are; ``route_scale`` multiplies them."""
 
     hidden: int
     n_experts: int
@@ -272,6 +347,9 @@ class RoutedMoESpec:
     shared_ff: Optional[int] = None
     shared_limit: Optional[float] = None
     kind: str = "routed_moe"
+    score: str = "softmax"
+    renormalize: bool = True
+    route_scale: float = 1.0
 
 
 @dataclass(frozen=True)

@@ -18,6 +18,10 @@
 // has no value: o = sum_u p_u v_u / (exp(-max) + sum_u p_u), the maximum taken over the scores and 0.  Value tables
 // (max_position, vd/2): the cached values were turned by their own positions (rope_kv.hip), and the head's sum is
 // turned back by the query's position, pair (a, b) -> (a cos + b sin, b cos - a sin), before it is stored.
+// softcap > 0: s_u <- softcap tanh(s_u / softcap).  keep_first > 0 (with a window): the first keep_first positions of
+// the sequence stay visible when the window has passed them; they are walked before the window's keys, at their own
+// positions.  sinks (one float32 a head): the extra term of the denominator is exp(sinks[h] - max) instead of
+// exp(0 - max); it is neither scaled nor capped.
 #include "common.h"
 
 #define GS_ATTN_MAX_D 256
@@ -29,7 +33,8 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
                                          int max_blocks, int page_size, int window, float scale, T* __restrict__ out,
                                          int nh, int nkv, int d, int vd, int chunk, int sink,
                                          const float* __restrict__ vcos, const float* __restrict__ vsin,
-                                         int interleaved) {
+                                         int interleaved, float softcap, int keep_first,
+                                         const float* __restrict__ sinks) {
   __shared__ float qs[GS_ATTN_MAX_D];
   __shared__ float ps[64];
   __shared__ long rowoff[64];
@@ -44,26 +49,39 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
 
   int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
   if (chunk > 0 && pos - pos % chunk > lo) lo = pos - pos % chunk;
+  // the kept first positions that the window has passed: [lo0, hi0), walked before the window's keys
+  int lo0 = chunk > 0 ? pos - pos % chunk : 0, hi0 = 0;
+  if (window > 0 && keep_first > 0) hi0 = keep_first < pos - window + 1 ? keep_first : pos - window + 1;
+  if (hi0 > lo) hi0 = lo;
   // with a sink the running maximum starts at the sink's score and the sum at its term
-  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
+  float m = sinks ? sinks[h] : (sink ? 0.f : -INFINITY), l = (sink || sinks) ? 1.f : 0.f;
   float acc[GS_ATTN_MAX_D / 64];
 #pragma unroll
   for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) acc[i] = 0.f;
 
-  for (int base = lo; base <= pos; base += 64) {
+  // two runs of keys: the kept first positions lo0 .. hi0 - 1 (where there are any), then lo .. pos
+  const bool kept = hi0 > lo0;
+  for (int base = kept ? lo0 : lo, last = kept ? hi0 - 1 : pos; base <= pos;) {
+    if (base > last) {
+      if (last == pos) break;
+      base = lo;
+      last = pos;
+      continue;
+    }
     int u = base + lane;
     float s = -INFINITY;
     long off = 0;
-    if (u <= pos) {
+    if (u <= last) {
       int page = bt[u / page_size];
       off = ((long)page * nkv + kvh) * page_size + u % page_size;
       const T* kr = kcache + off * d;
       float dot = 0.f;
       for (int j = 0; j < d; ++j) dot += qs[j] * to_f32(kr[j]);
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     float m_new = fmaxf(m, wave_max(s));
-    float p = u <= pos ? expf(s - m_new) : 0.f;
+    float p = u <= last ? expf(s - m_new) : 0.f;
     float alpha = expf(m - m_new);  // 0 on the first tile (m = -inf), since m_new is finite there
     l = l * alpha + wave_sum(p);
     m = m_new;
@@ -71,7 +89,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
     ps[lane] = p;
     rowoff[lane] = off;
     __syncthreads();
-    int nk = pos - base + 1 < 64 ? pos - base + 1 : 64;
+    int nk = last - base + 1 < 64 ? last - base + 1 : 64;
 #pragma unroll
     for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) {
       int j = lane + 64 * i;
@@ -81,6 +99,7 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
         acc[i] = a;
       }
     }
+    base += 64;
   }
   float inv = 1.0f / l;
   if (vcos) {
@@ -113,7 +132,8 @@ extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kca
                                     const int* positions, const int* seq_of_token, const int* block_table,
                                     int max_blocks, int page_size, int window, float scale, void* out, int ntok,
                                     int nh, int nkv, int d, int vd, int chunk, int sink, const float* vcos,
-                                    const float* vsin, int interleaved, hipStream_t stream) {
+                                    const float* vsin, int interleaved, float softcap, int keep_first,
+                                    const float* sinks, hipStream_t stream) {
   GS_REQUIRE(ntok >= 0 && nh > 0 && nkv > 0 && d > 0, "attention: bad sizes T=%d nh=%d nkv=%d d=%d", ntok, nh, nkv, d);
   GS_REQUIRE(nh % nkv == 0, "attention: %d query heads are no multiple of %d key heads", nh, nkv);
   GS_REQUIRE(d <= GS_ATTN_MAX_D, "attention: head width %d above the kernel's limit %d", d, GS_ATTN_MAX_D);
@@ -122,6 +142,8 @@ extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kca
   GS_REQUIRE(q_stride >= nh * d, "attention: q_stride %d below nh*d %d", q_stride, nh * d);
   GS_REQUIRE(vd > 0 && vd <= GS_ATTN_MAX_D, "attention: value width %d outside 1..%d", vd, GS_ATTN_MAX_D);
   GS_REQUIRE(chunk >= 0, "attention: bad chunk %d", chunk);
+  GS_REQUIRE(softcap >= 0.f && keep_first >= 0, "attention: bad cap %f or kept positions %d", (double)softcap, keep_first);
+  GS_REQUIRE(!(sink && sinks), "attention: the extra term is exp(0) or a head's own, not both");
   GS_REQUIRE((vcos == nullptr) == (vsin == nullptr) && (!vcos || vd % 2 == 0), "attention: value tables come together, for even widths");
   if (ntok == 0) return 0;
   dim3 grid(ntok, nh);
@@ -130,13 +152,13 @@ extern "C" int gs_attention_generic(const void* q, int q_stride, const void* kca
                                                               (const float*)vcache, positions, seq_of_token,
                                                               block_table, max_blocks, page_size, window, scale,
                                                               (float*)out, nh, nkv, d, vd, chunk, sink, vcos, vsin,
-                                                              interleaved);
+                                                              interleaved, softcap, keep_first, sinks);
   else if (dtype == GS_BF16)
     attention_generic_kernel<bf16><<<grid, 64, 0, stream>>>((const bf16*)q, q_stride, (const bf16*)kcache,
                                                              (const bf16*)vcache, positions, seq_of_token,
                                                              block_table, max_blocks, page_size, window, scale,
                                                              (bf16*)out, nh, nkv, d, vd, chunk, sink, vcos, vsin,
-                                                             interleaved);
+                                                             interleaved, softcap, keep_first, sinks);
   else
     GS_REQUIRE(false, "attention: unknown dtype %d", dtype);
   GS_LAUNCH_CHECK("attention_generic");

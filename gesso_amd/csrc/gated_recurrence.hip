@@ -1,0 +1,212 @@
+// Recurrences through a matrix state whose decay depends on the token, with or without the delta rule.
+//
+// Per sequence and head a state S (n x m, float32, in the request's slot) is advanced token by token:
+//
+//   S <- diag(a_t) S                      a_t: one number per (token, head), or one per (token, head, key channel)
+//   u_t = beta_t (v_t - S^T k_t)          with `delta` (the delta rule: what the state already answers to k_t is taken
+//                                         off the value before it is written);  u_t = v_t without
+//   S <- S + k_t u_t^T,   o_t = S^T (q_scale q_t)
+//
+// q_t, k_t (n values) and v_t (m values) are columns of a row buffer x (T, ld), float32 or bfloat16: q of head h at
+// [oq + (h / rep) n, ...), k at [ok + (h / rep) n, ...) (rep = H / qk_heads heads share one q and k), v at [ov + h m, ...).
+// The decays are float32 rows (T, lda): a_t of head h at [oa + h] or, per channel, at [oa + h n, ...); beta_t float32 at
+// [ob + h] of rows (T, ldb).  Nothing is rounded below float32 between the rows and the output (T, H m).
+//
+// gated_state_scan: one block per (sequence, head, tile of 64 value columns).  Thread (rg, jl) = (tid & 3, tid >> 2)
+// holds the state's rows rg, rg + 4, ... of column jl in registers; the four partial sums of a column (S^T k, S^T q)
+// are neighbours in a wavefront.  A step's tokens come through LDS eight at a time.  Every sum runs in one fixed
+// order, whatever the step's cut: a sequence fed whole, in portions or token by token leaves the same state and
+// outputs, bit for bit.  A step of single tokens is the same kernel with one token a block.
+//
+// delta_rule_prep: what the gated delta rule computes between its convolutions and the recurrence, in float32:
+//   q <- q / sqrt(sum q^2 + unit_eps) * q_scale,  k <- k / sqrt(sum k^2 + unit_eps)        per (token, q/k head), in place
+//   g = exp(-exp(A_log[h]) softplus(a + dt_bias[h])),  beta = sigmoid(b)                     per (token, head)
+// channel_decay: alpha = sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau), elementwise in place.
+#include "common.h"
+
+#define GR_TB 8          // tokens staged at once
+#define GR_COLS 64       // value columns a block
+
+__device__ __forceinline__ float gr_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+template <typename TI, int RMAX, bool VEC, bool DELTA>
+__global__ void __launch_bounds__(256)
+gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov, int rep, float q_scale,
+                        const float* __restrict__ decay, int lda, int oa, const float* __restrict__ beta, int ldb,
+                        int ob, float* __restrict__ state, const int* __restrict__ q_start,
+                        const int* __restrict__ slots, float* __restrict__ out, int H, int n, int m) {
+  constexpr int NMAX = 4 * RMAX;
+  __shared__ float qs[GR_TB][NMAX];
+  __shared__ float ks[GR_TB][NMAX];
+  __shared__ float al[VEC ? GR_TB : 1][VEC ? NMAX : 1];
+  __shared__ float vs[GR_TB][GR_COLS];
+  __shared__ float a1[GR_TB], bs[GR_TB];
+  const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * GR_COLS;
+  const int tid = threadIdx.x, rg = tid & 3, jl = tid >> 2, j = j0 + jl;
+  const int t0 = q_start[seq], t1 = q_start[seq + 1];
+  if (t1 <= t0) return;
+  const int hq = h / rep;
+  float* S = state + (((size_t)slots[seq] * H + h) * n) * m;
+  float s[RMAX];
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r) {
+    const int i = rg + 4 * r;
+    s[r] = (i < n && j < m) ? S[(size_t)i * m + j] : 0.f;
+  }
+  for (int tb = t0; tb < t1; tb += GR_TB) {
+    const int nb = t1 - tb < GR_TB ? t1 - tb : GR_TB;
+    __syncthreads();                                   // the batch before has been read
+    for (int idx = tid; idx < nb * n; idx += 256) {
+      const int tt = idx / n, i = idx - tt * n;
+      const TI* row = x + (size_t)(tb + tt) * ld;
+      qs[tt][i] = to_f32(row[oq + hq * n + i]) * q_scale;
+      ks[tt][i] = to_f32(row[ok + hq * n + i]);
+      if (VEC) al[tt][i] = decay[(size_t)(tb + tt) * lda + oa + h * n + i];
+    }
+    for (int idx = tid; idx < nb * GR_COLS; idx += 256) {
+      const int tt = idx / GR_COLS, c = idx - tt * GR_COLS;
+      vs[tt][c] = j0 + c < m ? to_f32(x[(size_t)(tb + tt) * ld + ov + h * m + j0 + c]) : 0.f;
+    }
+    if (tid < nb) {
+      if (!VEC) a1[tid] = decay[(size_t)(tb + tid) * lda + oa + h];
+      if (DELTA) bs[tid] = beta[(size_t)(tb + tid) * ldb + ob + h];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nb; ++tt) {
+      float u = vs[tt][jl];
+      const float a = VEC ? 0.f : a1[tt];
+      float answered = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) {
+        const int i = rg + 4 * r;
+        if (i < n) {
+          s[r] *= VEC ? al[tt][i] : a;
+          if (DELTA) answered = fmaf(s[r], ks[tt][i], answered);
+        }
+      }
+      if (DELTA) {
+        answered += __shfl_xor(answered, 1, 64);
+        answered += __shfl_xor(answered, 2, 64);
+        u = bs[tt] * (u - answered);
+      }
+      float part = 0.f;
+#pragma unroll
+      for (int r = 0; r < RMAX; ++r) {
+        const int i = rg + 4 * r;
+        if (i < n) {
+          s[r] = fmaf(ks[tt][i], u, s[r]);
+          part = fmaf(s[r], qs[tt][i], part);
+        }
+      }
+      part += __shfl_xor(part, 1, 64);
+      part += __shfl_xor(part, 2, 64);
+      if (rg == 0 && j < m) out[((size_t)(tb + tt) * H + h) * m + j] = part;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RMAX; ++r) {
+    const int i = rg + 4 * r;
+    if (i < n && j < m) S[(size_t)i * m + j] = s[r];
+  }
+}
+
+extern "C" int gs_gated_state_scan(const void* x, int dtype, int ld, int oq, int ok, int ov, int qk_heads, float q_scale,
+                                   const float* decay, int lda, int oa, int per_channel, const float* beta, int ldb,
+                                   int ob, float* state, const int* q_start, const int* slots, float* out, int nseq,
+                                   int H, int n, int m, hipStream_t stream) {
+  GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && m > 0, "gated_state_scan: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
+  GS_REQUIRE(n <= 256, "gated_state_scan: keys of %d features, the kernel holds up to 256", n);
+  GS_REQUIRE(qk_heads > 0 && H % qk_heads == 0, "gated_state_scan: %d heads do not share %d queries and keys evenly", H,
+             qk_heads);
+  GS_REQUIRE(H <= 65535 && (m + GR_COLS - 1) / GR_COLS <= 65535, "gated_state_scan: too many heads or value columns");
+  GS_REQUIRE(oq >= 0 && ok >= 0 && ov >= 0 && oq + qk_heads * n <= ld && ok + qk_heads * n <= ld && ov + H * m <= ld,
+             "gated_state_scan: q, k or v lie outside the rows of %d", ld);
+  GS_REQUIRE(decay && oa >= 0 && oa + (per_channel ? H * n : H) <= lda, "gated_state_scan: the decays lie outside their rows of %d", lda);
+  GS_REQUIRE(!beta || (ob >= 0 && ob + H <= ldb), "gated_state_scan: the write strengths lie outside their rows of %d", ldb);
+  if (nseq == 0) return 0;
+  dim3 grid(nseq, H, (m + GR_COLS - 1) / GR_COLS);
+  const int rep = H / qk_heads;
+#define GR_RUN(TI, R, V, D)                                                                                         \
+  gated_state_scan_kernel<TI, R, V, D><<<grid, 256, 0, stream>>>((const TI*)x, ld, oq, ok, ov, rep, q_scale, decay, \
+                                                                 lda, oa, beta, ldb, ob, state, q_start, slots, out, H, n, m)
+#define GR_RUN_R(TI, V, D)                   \
+  if (n <= 32) GR_RUN(TI, 8, V, D);          \
+  else if (n <= 64) GR_RUN(TI, 16, V, D);    \
+  else if (n <= 128) GR_RUN(TI, 32, V, D);   \
+  else GR_RUN(TI, 64, V, D)
+#define GR_RUN_T(TI)                                      \
+  if (per_channel && beta) { GR_RUN_R(TI, true, true); }  \
+  else if (per_channel) { GR_RUN_R(TI, true, false); }    \
+  else if (beta) { GR_RUN_R(TI, false, true); }           \
+  else { GR_RUN_R(TI, false, false); }
+  if (dtype == GS_F32) {
+    GR_RUN_T(float)
+  } else if (dtype == GS_BF16) {
+    GR_RUN_T(bf16)
+  } else {
+    GS_REQUIRE(false, "gated_state_scan: unknown dtype %d", dtype);
+  }
+#undef GR_RUN_T
+#undef GR_RUN_R
+#undef GR_RUN
+  GS_LAUNCH_CHECK("gated_state_scan");
+  return 0;
+}
+
+// One block of 256 threads per token: a wavefront per q or k head in turn, then the heads' gates.
+//   c (T, ldc) float32: q heads at [0, G n), k heads at [G n, 2 G n), normed in place
+//   rows (T, ldr): the decay's product at [oa + h], the write strength's at [obeta + h]
+//   gates (T, 2 H) float32: g at [h], beta at [H + h]
+template <typename TR>
+__global__ void __launch_bounds__(256)
+delta_rule_prep_kernel(float* __restrict__ c, int ldc, int G, int n, float q_scale, float unit_eps,
+                       const TR* __restrict__ rows, int ldr, int oa, int obeta, const float* __restrict__ a_log,
+                       const float* __restrict__ dt_bias, float* __restrict__ gates, int H) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int u = wave; u < 2 * G; u += 4) {
+    float* v = c + (size_t)t * ldc + (size_t)u * n;
+    float ss = 0.f;
+    for (int i = lane; i < n; i += 64) ss += v[i] * v[i];
+    ss = wave_sum(ss);
+    const float inv = (u < G ? q_scale : 1.f) / sqrtf(ss + unit_eps);
+    for (int i = lane; i < n; i += 64) v[i] *= inv;
+  }
+  for (int h = threadIdx.x; h < H; h += 256) {
+    const float a = to_f32(rows[(size_t)t * ldr + oa + h]), b = to_f32(rows[(size_t)t * ldr + obeta + h]);
+    gates[(size_t)t * 2 * H + h] = expf(-expf(a_log[h]) * gr_softplus(a + dt_bias[h]));
+    gates[(size_t)t * 2 * H + H + h] = 1.f / (1.f + expf(-b));
+  }
+}
+
+extern "C" int gs_delta_rule_prep(float* c, int ldc, int G, int n, float q_scale, float unit_eps, const void* rows,
+                                  int rows_dtype, int ldr, int oa, int obeta, const float* a_log, const float* dt_bias,
+                                  float* gates, int T, int H, hipStream_t stream) {
+  GS_REQUIRE(T >= 0 && G > 0 && n > 0 && H > 0 && 2 * G * n <= ldc, "delta_rule_prep: bad sizes T=%d G=%d n=%d H=%d ldc=%d",
+             T, G, n, H, ldc);
+  GS_REQUIRE(oa >= 0 && obeta >= 0 && oa + H <= ldr && obeta + H <= ldr, "delta_rule_prep: the gates' products lie outside the rows of %d", ldr);
+  GS_REQUIRE(unit_eps >= 0.f, "delta_rule_prep: bad eps");
+  if (T == 0) return 0;
+  if (rows_dtype == GS_F32)
+    delta_rule_prep_kernel<float><<<T, 256, 0, stream>>>(c, ldc, G, n, q_scale, unit_eps, (const float*)rows, ldr, oa,
+                                                          obeta, a_log, dt_bias, gates, H);
+  else if (rows_dtype == GS_BF16)
+    delta_rule_prep_kernel<bf16><<<T, 256, 0, stream>>>(c, ldc, G, n, q_scale, unit_eps, (const bf16*)rows, ldr, oa,
+                                                         obeta, a_log, dt_bias, gates, H);
+  else
+    GS_REQUIRE(false, "delta_rule_prep: unknown dtype %d", rows_dtype);
+  GS_LAUNCH_CHECK("delta_rule_prep");
+  return 0;
+}
+
+__global__ void channel_decay_kernel(float* __restrict__ z, long total, float inv_tau) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) z[i] = expf(-gr_softplus(-z[i]) * inv_tau);
+}
+
+extern "C" int gs_channel_decay(float* z, long total, float tau, hipStream_t stream) {
+  GS_REQUIRE(total >= 0 && tau > 0.f, "channel_decay: bad sizes or tau");
+  if (total == 0) return 0;
+  channel_decay_kernel<<<gs_ceil_div(total, 256), 256, 0, stream>>>(z, total, 1.f / tau);
+  GS_LAUNCH_CHECK("channel_decay");
+  return 0;
+}

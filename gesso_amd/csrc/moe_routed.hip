@@ -1,7 +1,8 @@
 // A mixture of gated feed-forwards chosen by a router over the token's own features.
 //
-//   z = W_r x (float32), s = softmax(z) over all router outputs; the `top` outputs with the largest s + correction are
-//   chosen; the chosen ones' weights are their s divided by the sum of the chosen s (+ 1e-20).  Outputs e >= E name no
+//   z = W_r x (float32), s = softmax(z) over all router outputs (or, with score_fn 1, s = sigmoid(z), each output for
+//   itself); the `top` outputs with the largest s + correction are chosen; the chosen ones' weights are their s divided
+//   by the sum of the chosen s (+ 1e-20), or, without `renorm`, their s as they are; both times route_scale.  Outputs e >= E name no
 //   expert with weights: such an "identity expert" gives back its input.  An expert is
 //     g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = W_down (g sigmoid(alpha g) (u + 1)).
 //   Expert weights lie stacked: gate_up (E, 2F, H) (a gate's rows, then the up rows), down (E, H, F).
@@ -38,24 +39,33 @@ __device__ __forceinline__ void stage_row(float* xs, const T* __restrict__ row, 
   }
 }
 
-// One wavefront, from a token's logits in `z` (LDS, EA floats; `cs` as many, `chosen` top ints): softmax, the `top`
-// largest corrected scores (of equal ones the lowest index), the chosen ones' weights.
+// One wavefront, from a token's logits in `z` (LDS, EA floats; `cs` as many, `chosen` top ints): the scores (softmax
+// over the outputs, or each output's sigmoid), the `top` largest corrected scores (of equal ones the lowest index), the
+// chosen ones' weights.
 __device__ __forceinline__ void route_from_logits(float* z, float* cs, int* chosen, const float* __restrict__ correction,
                                                   int top, int EA, int lane, int t, int* __restrict__ choice,
-                                                  float* __restrict__ weight) {
-  float m = -INFINITY;
-  for (int e = lane; e < EA; e += 64) m = fmaxf(m, z[e]);
-  m = wave_max(m);
-  float sum = 0.f;
-  for (int e = lane; e < EA; e += 64) {
-    const float p = expf(z[e] - m);
-    z[e] = p;
-    sum += p;
-  }
-  sum = wave_sum(sum);
-  for (int e = lane; e < EA; e += 64) {
-    z[e] = z[e] / sum;
-    cs[e] = z[e] + (correction ? correction[e] : 0.f);
+                                                  float* __restrict__ weight, int score_fn, int renorm,
+                                                  float route_scale) {
+  if (score_fn == 1) {
+    for (int e = lane; e < EA; e += 64) {
+      z[e] = 1.f / (1.f + expf(-z[e]));
+      cs[e] = z[e] + (correction ? correction[e] : 0.f);
+    }
+  } else {
+    float m = -INFINITY;
+    for (int e = lane; e < EA; e += 64) m = fmaxf(m, z[e]);
+    m = wave_max(m);
+    float sum = 0.f;
+    for (int e = lane; e < EA; e += 64) {
+      const float p = expf(z[e] - m);
+      z[e] = p;
+      sum += p;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < EA; e += 64) {
+      z[e] = z[e] / sum;
+      cs[e] = z[e] + (correction ? correction[e] : 0.f);
+    }
   }
   // the largest choice score `top` times over; of equal scores the lowest index
   float picked = 0.f;
@@ -82,7 +92,7 @@ __device__ __forceinline__ void route_from_logits(float* z, float* cs, int* chos
     chosen[k] = cand;
     picked += z[cand];
   }
-  const float inv = 1.f / (picked + 1e-20f);
+  const float inv = (renorm ? 1.f / (picked + 1e-20f) : 1.f) * route_scale;
   for (int k = lane; k < top; k += 64) {
     choice[(size_t)t * top + k] = chosen[k];
     weight[(size_t)t * top + k] = z[chosen[k]] * inv;
@@ -92,7 +102,8 @@ __device__ __forceinline__ void route_from_logits(float* z, float* cs, int* chos
 template <typename T, typename TW>
 __global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ x, int ldx, const TW* __restrict__ wr,
                                                          const float* __restrict__ correction, int top, int EA, int H,
-                                                         int* __restrict__ choice, float* __restrict__ weight) {
+                                                         int* __restrict__ choice, float* __restrict__ weight,
+                                                         int score_fn, int renorm, float route_scale) {
   extern __shared__ float mr_sh[];           // H floats of the row, EA logits, EA choice scores, top chosen outputs
   float* xs = mr_sh;
   float* z = mr_sh + H;
@@ -144,7 +155,7 @@ __global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ 
   }
   __syncthreads();
   if (wave != 0) return;
-  route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight);
+  route_from_logits(z, cs, chosen, correction, top, EA, lane, t, choice, weight, score_fn, renorm, route_scale);
 }
 
 template <typename TI, typename TO>
@@ -290,7 +301,9 @@ static int moe_routed_blocks_y(int outputs, int tokens) {
 }
 
 extern "C" int gs_moe_router(const void* x, int dtype, int ldx, const void* wr, int w_dtype, const float* correction,
-                             int top, int EA, int H, int* choice, float* weight, int ntok, hipStream_t stream) {
+                             int top, int EA, int H, int* choice, float* weight, int ntok, int score_fn, int renorm,
+                             float route_scale, hipStream_t stream) {
+  GS_REQUIRE(score_fn == 0 || score_fn == 1, "moe_router: scores are a softmax (0) or sigmoids (1), not %d", score_fn);
   GS_REQUIRE(ntok >= 0 && top > 0 && EA >= top && H > 0 && ldx >= H, "moe_router: bad sizes T=%d top=%d outputs=%d H=%d", ntok, top, EA, H);
   const size_t lds = ((size_t)H + 2 * (size_t)EA + (size_t)top) * sizeof(float);
   GS_REQUIRE(lds <= 65536, "moe_router: rows of %d and %d outputs are more than the kernel stages", H, EA);
@@ -299,13 +312,13 @@ extern "C" int gs_moe_router(const void* x, int dtype, int ldx, const void* wr, 
   const int threads = 64 * (gs_ceil_div(EA, 4) < 16 ? (gs_ceil_div(EA, 4) < 4 ? 4 : gs_ceil_div(EA, 4)) : 16);
   if (dtype == GS_F32 && w_dtype == GS_F32)
     moe_router_kernel<float, float><<<ntok, threads, lds, stream>>>((const float*)x, ldx, (const float*)wr, correction, top,
-                                                                EA, H, choice, weight);
+                                                                EA, H, choice, weight, score_fn, renorm, route_scale);
   else if (dtype == GS_BF16 && w_dtype == GS_BF16)
     moe_router_kernel<bf16, bf16><<<ntok, threads, lds, stream>>>((const bf16*)x, ldx, (const bf16*)wr, correction, top, EA, H,
-                                                              choice, weight);
+                                                              choice, weight, score_fn, renorm, route_scale);
   else if (dtype == GS_BF16 && w_dtype == GS_F32)
     moe_router_kernel<bf16, float><<<ntok, threads, lds, stream>>>((const bf16*)x, ldx, (const float*)wr, correction, top, EA,
-                                                               H, choice, weight);
+                                                               H, choice, weight, score_fn, renorm, route_scale);
   else
     GS_REQUIRE(false, "moe_router: unsupported types %d %d", dtype, w_dtype);
   GS_LAUNCH_CHECK("moe_router");

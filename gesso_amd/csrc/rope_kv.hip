@@ -12,6 +12,10 @@
 // A value head may be vd wide instead of d (the row is then (nh + nkv) d + nkv vd wide, the value cache
 // (num_pages, nkv, page_size, vd)), and with value tables (max_position, vd/2) the values are cached turned by
 // their own position over their whole width, in the same layout of pairs; whoever sums them turns the sum back.
+// The rows may be wider than q|k|v (`ld` values apart: further products of the same input stand behind them).
+// `plain_norm`: q and k are divided by their root mean square without a weight (a turn keeps a head's sum of squares,
+// so the same numbers come out whether the division stands before or after it).  `v_first` (rows `ldf` apart, the value
+// heads from column 0 on) with `mix` (one float on the device): the values are cached as (1 - mix) v + mix v_first.
 // One wave per (token, head).  All arithmetic float32.
 #include "common.h"
 
@@ -22,14 +26,16 @@ __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restri
                                       const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
                                       int max_blocks, int page_size, T* __restrict__ kcache, T* __restrict__ vcache,
                                       int ntok, int nh, int nkv, int d, int write_kv, int vd,
-                                      const float* __restrict__ vcos, const float* __restrict__ vsin) {
+                                      const float* __restrict__ vcos, const float* __restrict__ vsin, int ld,
+                                      int plain_norm, const T* __restrict__ v_first, int ldf,
+                                      const float* __restrict__ mix) {
   int lane = threadIdx.x & 63;
   int heads = nh + 2 * nkv;
   long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (unit >= (long)ntok * heads) return;
   int t = (int)(unit / heads);
   int hh = (int)(unit - (long)t * heads);
-  const size_t row_len = (size_t)(nh + nkv) * d + (size_t)nkv * vd;
+  const size_t row_len = (size_t)ld;
   const bool is_v = hh >= nh + nkv;
   T* x = qkv + (size_t)t * row_len + (is_v ? (size_t)(nh + nkv) * d + (size_t)(hh - nh - nkv) * vd : (size_t)hh * d);
   int pos = positions[t];
@@ -42,7 +48,13 @@ __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restri
     T* base = is_v ? vcache : kcache;
     dst = base + (((size_t)page * nkv + kvh) * page_size + pos % page_size) * (is_v ? vd : d);
   }
-  if (is_v) {  // v: copy, or turn by the position over the whole width
+  if (is_v) {  // v: copy, blend with another layer's values, or turn by the position over the whole width
+    if (v_first) {
+      const float lam = mix[0];
+      const T* f = v_first + (size_t)t * ldf + (size_t)(hh - nh - nkv) * vd;
+      for (int j = lane; j < vd; j += 64) dst[j] = from_f32<T>((1.f - lam) * to_f32(x[j]) + lam * to_f32(f[j]));
+      return;
+    }
     if (!vcos) {
       for (int j = lane; j < vd; j += 64) dst[j] = x[j];
       return;
@@ -60,7 +72,7 @@ __global__ void qknorm_rope_kv_kernel(T* __restrict__ qkv, const float* __restri
 
   const float* w = hh < nh ? qw : kw;
   float inv = 1.f;
-  if (w) {
+  if (w || plain_norm) {
     float ss = 0.f;
     for (int j = lane; j < d; j += 64) {
       float v = to_f32(x[j]);
@@ -152,7 +164,8 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
                                  const float* cos_t, const float* sin_t, int rotary_dim, int interleaved,
                                  int max_position, const int* positions, const int* seq_of_token, const int* block_table,
                                  int max_blocks, int page_size, void* kcache, void* vcache, int ntok, int nh, int nkv,
-                                 int d, int write_kv, int vd, const float* vcos, const float* vsin,
+                                 int d, int write_kv, int vd, const float* vcos, const float* vsin, int ld,
+                                 int plain_norm, const void* v_first, int ldf, const float* mix,
                                  hipStream_t stream) {
   GS_REQUIRE(vd > 0, "qknorm_rope_kv: values of width %d", vd);
   GS_REQUIRE((vcos == nullptr) == (vsin == nullptr), "qknorm_rope_kv: the value tables come together");
@@ -165,9 +178,15 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
   GS_REQUIRE(page_size > 0 && max_blocks > 0, "qknorm_rope_kv: bad page_size %d or max_blocks %d", page_size,
              max_blocks);
   GS_REQUIRE((qw == nullptr) == (kw == nullptr), "qknorm_rope_kv: q and k norm weights come together");
+  const int narrow = (nh + nkv) * d + nkv * vd;
+  if (ld == 0) ld = narrow;
+  GS_REQUIRE(ld >= narrow, "qknorm_rope_kv: rows of %d values do not hold q, k and v (%d)", ld, narrow);
+  GS_REQUIRE(!(plain_norm && qw), "qknorm_rope_kv: a head norm has a weight or none");
+  GS_REQUIRE((v_first == nullptr) == (mix == nullptr) && (!v_first || (ldf >= nkv * vd && !vcos)),
+             "qknorm_rope_kv: blended values need the other values (rows of at least %d) and the share", nkv * vd);
   if (ntok == 0) return 0;
   long units = (long)ntok * (nh + 2 * nkv);
-  const bool vec = !interleaved && vd == d && !vcos && rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
+  const bool vec = ld == narrow && !plain_norm && !v_first && !interleaved && vd == d && !vcos && rotary_dim == d && (d == 16 || d == 32 || d == 64 || d == 128) && (dtype == GS_F32 || dtype == GS_BF16) &&
                    ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)kcache & 15) == 0 && ((uintptr_t)vcache & 15) == 0 &&
                    ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 && ((uintptr_t)qw & 15) == 0 &&
                    ((uintptr_t)kw & 15) == 0;
@@ -195,7 +214,8 @@ extern "C" int gs_qknorm_rope_kv(void* qkv, int dtype, const float* qw, const fl
 #define GS_RUN(T)                                                                                               \
   qknorm_rope_kv_kernel<T><<<blocks, 256, 0, stream>>>((T*)qkv, qw, kw, eps, cos_t, sin_t, rotary_dim, interleaved, positions, \
                                                        seq_of_token, block_table, max_blocks, page_size,        \
-                                                       (T*)kcache, (T*)vcache, ntok, nh, nkv, d, write_kv, vd, vcos, vsin)
+                                                       (T*)kcache, (T*)vcache, ntok, nh, nkv, d, write_kv, vd, vcos, vsin, \
+                                                       ld, plain_norm, (const T*)v_first, ldf, mix)
   if (dtype == GS_F32)
     GS_RUN(float);
   else if (dtype == GS_BF16)

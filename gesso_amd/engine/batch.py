@@ -80,6 +80,9 @@ class BatchContext:
         self._storage = storage
         self._tiles = None
         self._segments = None
+        # what one part of a step leaves for a later part of the same step (values that later layers blend with
+        # theirs); empty at a step's start, gone at its end
+        self.shared = {}
 
     def cache_view(self, call: int):
         return self._storage.view(call, self.block_tables)

@@ -192,6 +192,6 @@ def load() -> ctypes.CDLL:
                 continue
             f.restype, f.argtypes = res, args
         _lib.gs_last_error.restype = ctypes.c_char_p
-        if _lib.gs_abi_version() != 11:
+        if _lib.gs_abi_version() != 12:
             raise KernelError("the HIP extension has another interface version; build it again")
         return _lib

@@ -315,16 +315,26 @@ def _value_tables(vcos, vsin, vd):
 
 def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions, seq_of_token, block_table,
                    page_size, kcache, vcache, nh, nkv, d, write_kv=True, layout: str = "half", vd: int = None,
-                   vcos=None, vsin=None) -> None:
+                   vcos=None, vsin=None, plain_norm: bool = False, v_first=None, mix=None) -> None:
     """Head norm and rotation of q (in place) and k; k and v written into the pages.  ``layout``: which features
     form a rotation pair, ``"half"`` (i, i + rotary_dim/2) or ``"interleaved"`` (2i, 2i + 1).  ``vd``: the width of
     a value head where it is not ``d``; ``vcos``, ``vsin`` ``(P, vd/2)``: the values are cached turned by their
-    position over their whole width."""
+    position over their whole width.  The rows may hold more columns behind q|k|v.  ``plain_norm``: q and k are divided
+    by their root mean square, no weight.  ``v_first (T, >= nkv vd)`` (a range of columns of wider rows will do) with
+    ``mix`` (one float32 on the device): the values are cached as ``(1 - mix) v + mix v_first``."""
     _need(layout in ROPE_LAYOUTS, f"qknorm_rope_kv: pairs are laid out 'half' or 'interleaved', not {layout!r}")
-    _dev(qkv, q_weight, k_weight, cos, sin, positions, seq_of_token, block_table, kcache, vcache)
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, seq_of_token, block_table, kcache, vcache, mix)
     vd = d if vd is None else int(vd)
     T = qkv.shape[0]
-    _need(qkv.shape == (T, (nh + nkv) * d + nkv * vd), "qknorm_rope_kv: qkv must be (T, (nh + nkv) d + nkv vd)")
+    _need(qkv.dim() == 2 and qkv.shape[1] >= (nh + nkv) * d + nkv * vd, "qknorm_rope_kv: rows hold at least (nh + nkv) d + nkv vd values")
+    _need(not (plain_norm and q_weight is not None), "qknorm_rope_kv: a head norm has a weight or none")
+    _need((v_first is None) == (mix is None), "qknorm_rope_kv: the other values and their share come together")
+    ldf = 0
+    if v_first is not None:
+        _need(v_first.is_cuda and v_first.dim() == 2 and v_first.shape == (T, nkv * vd) and v_first.stride(1) == 1
+              and v_first.dtype == qkv.dtype and mix.dtype == torch.float32 and mix.numel() == 1,
+              "qknorm_rope_kv: the other values are (T, nkv vd) of the rows' type, their share one float32")
+        ldf = v_first.stride(0) if T > 1 else nkv * vd
     for w in (q_weight, k_weight):
         _need(w is None or (w.dtype == torch.float32 and w.shape == (d,)), "qknorm_rope_kv: head norm weight must be float32 (d,)")
     max_pos = 0
@@ -346,17 +356,22 @@ def qknorm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, positions
                                    _p(positions), _p(seq_of_token),
                                    _p(block_table), c_int(block_table.shape[1]), c_int(page_size), _p(kcache),
                                    _p(vcache), c_int(T), c_int(nh), c_int(nkv), c_int(d),
-                                   c_int(1 if write_kv else 0), c_int(vd), _p(vcos), _p(vsin), _stream()))
+                                   c_int(1 if write_kv else 0), c_int(vd), _p(vcos), _p(vsin), c_int(qkv.shape[1]),
+                                   c_int(1 if plain_norm else 0), _p(v_first), c_int(ldf), _p(mix), _stream()))
 
 
 def attention_generic(q, q_stride, kcache, vcache, positions, seq_of_token, block_table, page_size, window, scale,
                       nh, nkv, d, ntok, out: torch.Tensor = None, vd: int = None, chunk: int = None, sink: bool = False,
-                      vcos=None, vsin=None, layout: str = "half") -> torch.Tensor:
+                      vcos=None, vsin=None, layout: str = "half", softcap: float = None, keep_first: int = 0,
+                      sinks=None) -> torch.Tensor:
     """Causal GQA over the paged cache, any sizes; ``q`` rows are ``q_stride`` apart.  ``vd``: the width of a value
     head where it is not ``d``; ``chunk``: a query sees only the keys of its own run of ``chunk`` positions;
     ``sink``: one more term ``exp(0)`` in the softmax's denominator; ``vcos``, ``vsin``: the cached values are turned
-    by their positions, and a head's sum is turned back by the query's (pairs laid out as ``layout`` says)."""
-    _dev(q, kcache, vcache, positions, seq_of_token, block_table, out)
+    by their positions, and a head's sum is turned back by the query's (pairs laid out as ``layout`` says);
+    ``softcap``: scores become ``softcap tanh(score / softcap)``; ``keep_first``: with a window, the sequence's first
+    positions that stay visible beyond it; ``sinks (nh,)`` float32: the extra term is ``exp(sinks[h])``."""
+    _dev(q, kcache, vcache, positions, seq_of_token, block_table, out, sinks)
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (nh,)), "attention: sinks must be float32 (nh,)")
     vd = d if vd is None else int(vd)
     _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention: q is too small")
     _need(kcache.dtype == q.dtype and vcache.dtype == q.dtype, "cache and activations differ in type")
@@ -375,7 +390,8 @@ def attention_generic(q, q_stride, kcache, vcache, positions, seq_of_token, bloc
                                       c_int(page_size), c_int(window or 0), c_float(scale), _p(out), c_int(ntok),
                                       c_int(nh), c_int(nkv), c_int(d), c_int(vd), c_int(chunk or 0),
                                       c_int(1 if sink else 0), _p(vcos), _p(vsin),
-                                      c_int(1 if layout == "interleaved" else 0), _stream()))
+                                      c_int(1 if layout == "interleaved" else 0), c_float(softcap or 0.0),
+                                      c_int(keep_first or 0), _p(sinks), _stream()))
     return out
 
 
@@ -1416,10 +1432,15 @@ def ssd_scan(xbc, rows, odt: int, dt_bias, a_log, d_skip, state, q_start, slots,
 
 # ---------------------------------------------------------------------- feed-forwards chosen by a router
 
-def moe_router(x, router, correction, top: int):
-    """Scores = softmax of ``router (EA, H) @ x[t]`` in float32; the ``top`` outputs with the largest score +
-    ``correction`` are chosen (of equal ones the lowest index), their weights are their scores divided by the chosen
-    scores' sum (+ 1e-20).  Returns ``(choice int32 (T, top), weight float32 (T, top))``."""
+ROUTER_SCORES = {"softmax": 0, "sigmoid": 1}
+
+
+def moe_router(x, router, correction, top: int, score: str = "softmax", renormalize: bool = True, scale: float = 1.0):
+    """Scores = softmax (or, with ``score="sigmoid"``, each output's sigmoid) of ``router (EA, H) @ x[t]`` in float32; the
+    ``top`` outputs with the largest score + ``correction`` are chosen (of equal ones the lowest index), their weights
+    are their scores divided by the chosen scores' sum (+ 1e-20) (as they are without ``renormalize``), times ``scale``.
+    Returns ``(choice int32 (T, top), weight float32 (T, top))``."""
+    _need(score in ROUTER_SCORES, f"moe_router: scores are one of {sorted(ROUTER_SCORES)}, not {score!r}")
     _dev(router, correction)
     ldx = _cols(x, "moe_router")
     T, H = x.shape
@@ -1429,7 +1450,7 @@ def moe_router(x, router, correction, top: int):
     choice = torch.empty((T, top), dtype=torch.int32, device=x.device)
     weight = torch.empty((T, top), dtype=torch.float32, device=x.device)
     _check(lib().gs_moe_router(_p(x), _dt(x), ldx, _p(router), _dt(router), _p(correction), top, EA, H, _p(choice),
-                               _p(weight), T, _stream()))
+                               _p(weight), T, ROUTER_SCORES[score], 1 if renormalize else 0, float(scale), _stream()))
     return choice, weight
 
 
@@ -1501,3 +1522,116 @@ def moe_routed_grouped(x, choice, weight, gate_up, down, limit: float, alpha: fl
     _check(L.gs_moe_group_gemm(_p(inner), F, None, _p(down), _p(ys), F32, H, _p(tiles), max_tiles, _p(n_tiles), H, F, 0, s))
     _check(L.gs_moe_routed_combine(_p(ys), _p(place_of), _p(weight), top, _p(x), ldx, _p(shared), _p(y), _dt(y), T, H, s))
     return y
+
+
+# ---------------------------------------------------------------------- layer norm, the sum of two normed branches, a gate on rows
+
+def add_layernorm(res: torch.Tensor, delta, weight: torch.Tensor, bias, eps: float, out_dtype, rows=None,
+                  out: torch.Tensor = None) -> torch.Tensor:
+    """``res += delta`` (when given and no ``rows``), then ``out = (res - mean) / sqrt(var + eps) * weight + bias`` with
+    the variance the mean of the squared deviations.  ``rows`` (int32) picks source rows; then ``res`` is not written."""
+    _dev(res, delta, weight, bias, rows, out)
+    _need(res.dtype == torch.float32 and res.dim() == 2, "add_layernorm: the residual stream is float32 (T, H)")
+    T, H = res.shape
+    for v in (weight, bias):
+        _need(v is None or (v.dtype == torch.float32 and v.shape == (H,)), "add_layernorm: weight and bias must be float32 (H,)")
+    _need(weight is not None, "add_layernorm: a weight")
+    _need(delta is None or delta.shape == res.shape, "add_layernorm: delta must have the stream's shape")
+    n_out = T
+    if rows is not None:
+        _i32(rows, what="rows")
+        n_out = rows.numel()
+    if out is None:
+        out = torch.empty((n_out, H), dtype=out_dtype, device=res.device)
+    _need(out.shape == (n_out, H) and out.dtype == out_dtype, "add_layernorm: out has the wrong shape or type")
+    _check(lib().gs_add_layernorm(_p(res), _p(delta), _dt(delta) if delta is not None else _dt(out), _p(weight), _p(bias),
+                                  float(eps), _p(out), _dt(out), _p(rows), n_out, H, _stream()))
+    return out
+
+
+def normed_pair_sum(a, wa, sa: float, b, wb, sb: float, eps: float, out_dtype) -> torch.Tensor:
+    """``sa * rms(a) * wa + sb * rms(b) * wb`` row by row, ``rms(x) = x / sqrt(mean(x^2) + eps)``: ``a``, ``b`` float32
+    ``(T, W)`` (two branches' last products), ``wa``, ``wb`` float32 ``(W,)``; one rounding, to ``out_dtype``."""
+    _dev(a, b, wa, wb)
+    _need(a.dtype == torch.float32 and b.dtype == torch.float32 and a.dim() == 2 and a.shape == b.shape,
+          "normed_pair_sum: the branches' rows are float32 (T, W)")
+    T, W = a.shape
+    for w in (wa, wb):
+        _need(w.dtype == torch.float32 and w.shape == (W,), "normed_pair_sum: weights must be float32 (W,)")
+    out = torch.empty((T, W), dtype=out_dtype, device=a.device)
+    _check(lib().gs_normed_pair_sum(_p(a), _p(b), _p(wa), _p(wb), float(eps), float(sa), float(sb), _p(out), _dt(out), T, W,
+                                    _stream()))
+    return out
+
+
+def gated_rows(o, gate_rows, og: int, gate: str = "sigmoid") -> torch.Tensor:
+    """``o (T, W)`` times ``sigmoid`` or ``silu`` of the gate, which stands in ``gate_rows (T, ldg)`` from column ``og``
+    on; float32 arithmetic, the result in the rows' type."""
+    _dev(o, gate_rows)
+    _need(o.dim() == 2 and gate_rows.dim() == 2 and gate_rows.shape[0] == o.shape[0] and gate_rows.dtype == o.dtype,
+          "gated_rows: rows (T, W) and gate rows (T, ldg) of one type")
+    _need(gate in _GATES, f"gated_rows: the gate is 'sigmoid' or 'silu', not {gate!r}")
+    T, W = o.shape
+    out = torch.empty_like(o)
+    _check(lib().gs_gated_rows(_p(o), _p(gate_rows), _dt(o), gate_rows.shape[1], og, _GATES[gate], _p(out), T, W, _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- recurrences with token-dependent decay
+
+GATED_STATE_MAX_KEY = 256
+
+
+def gated_state_scan(x, oq: int, ok: int, ov: int, H: int, qk_heads: int, n: int, m: int, decay, oa: int,
+                     per_channel: bool, state, q_start, slots, nseq: int, q_scale: float = 1.0, beta=None, ob: int = 0,
+                     out: torch.Tensor = None) -> torch.Tensor:
+    """Per sequence and head ``S <- diag(a_t) S; u = beta_t (v_t - S^T k_t)`` (``u = v_t`` without ``beta``);
+    ``S <- S + k_t u^T; o_t = S^T (q_scale q_t)``.
+
+    ``x (T, ld)`` float32 or bfloat16 holds q of head ``h`` at ``[oq + (h // (H / qk_heads)) n, ...)``, k likewise from
+    ``ok``, v at ``[ov + h m, ...)``.  ``decay`` float32 rows: ``a_t`` of head ``h`` at ``[oa + h]``, or with
+    ``per_channel`` one a key channel at ``[oa + h n, ...)``.  ``beta`` float32 rows with head ``h`` at ``[ob + h]``.
+    ``state (slots, H, n, m)`` float32 is read and advanced.  Returns ``(T, H m)`` float32."""
+    _dev(x, decay, beta, state, q_start, slots, out)
+    _need(x.dim() == 2 and decay.dim() == 2 and decay.dtype == torch.float32 and decay.shape[0] == x.shape[0],
+          "gated_state_scan: rows (T, ld) and float32 decay rows (T, lda)")
+    _need(beta is None or (beta.dim() == 2 and beta.dtype == torch.float32 and beta.shape[0] == x.shape[0]),
+          "gated_state_scan: the write strengths are float32 rows (T, ldb)")
+    T, ld = x.shape
+    _need(n <= GATED_STATE_MAX_KEY, f"gated_state_scan: keys of {n} features, the kernel holds up to {GATED_STATE_MAX_KEY}")
+    _need(state.dtype == torch.float32 and state.dim() == 4 and state.shape[1:] == (H, n, m),
+          "gated_state_scan: state must be float32 (slots, H, n, m)")
+    _i32(q_start, nseq + 1, "q_start")
+    _i32(slots, nseq, "slots")
+    if out is None:
+        out = torch.empty((T, H * m), dtype=torch.float32, device=x.device)
+    _need(out.shape == (T, H * m) and out.dtype == torch.float32, "gated_state_scan: out must be float32 (T, H m)")
+    _check(lib().gs_gated_state_scan(_p(x), _dt(x), ld, oq, ok, ov, qk_heads, float(q_scale), _p(decay), decay.shape[1], oa,
+                                     1 if per_channel else 0, _p(beta), beta.shape[1] if beta is not None else 0, ob,
+                                     _p(state), _p(q_start), _p(slots), _p(out), nseq, H, n, m, _stream()))
+    return out
+
+
+def delta_rule_prep(c, G: int, n: int, q_scale: float, unit_eps: float, rows, oa: int, ob: int, a_log, dt_bias, H: int):
+    """In place on ``c (T, >= 2 G n)`` float32: each of the ``G`` q heads (first) and ``G`` k heads (behind them) becomes
+    ``x / sqrt(sum(x^2) + unit_eps)``, q also times ``q_scale``.  Returns float32 ``(T, 2 H)``:
+    ``exp(-exp(a_log) softplus(rows[:, oa + h] + dt_bias))`` in the first ``H`` columns, ``sigmoid(rows[:, ob + h])`` in
+    the others."""
+    _dev(c, rows, a_log, dt_bias)
+    T = c.shape[0]
+    _need(c.dtype == torch.float32 and c.dim() == 2 and c.shape[1] >= 2 * G * n, "delta_rule_prep: float32 rows that hold q and k")
+    _need(rows.dim() == 2 and rows.shape[0] == T, "delta_rule_prep: the gates' products are rows (T, ld)")
+    for v in (a_log, dt_bias):
+        _need(v.dtype == torch.float32 and v.shape == (H,), "delta_rule_prep: a_log and dt_bias must be float32 (H,)")
+    gates = torch.empty((T, 2 * H), dtype=torch.float32, device=c.device)
+    _check(lib().gs_delta_rule_prep(_p(c), c.shape[1], G, n, float(q_scale), float(unit_eps), _p(rows), _dt(rows),
+                                    rows.shape[1], oa, ob, _p(a_log), _p(dt_bias), _p(gates), T, H, _stream()))
+    return gates
+
+
+def channel_decay(z, tau: float) -> torch.Tensor:
+    """In place on float32 ``z``: ``sigmoid(z)^(1/tau)``."""
+    _dev(z)
+    _need(z.dtype == torch.float32, "channel_decay: float32 values")
+    _check(lib().gs_channel_decay(_p(z), z.numel(), float(tau), _stream()))
+    return z

@@ -106,6 +106,7 @@ class Model:
         """The embedding and every scheduled block: the residual stream as the last block leaves it (what is still
         pending is added by the norm that follows)."""
         rt = self.rt
+        ctx.shared = {}          # what a part of this step leaves for a later one (a context may serve several runs)
         # the norm that reads the stream after the i-th scheduled block: the next block's first, then the final one
         # (``first_norm`` and ``row_weight`` are the optional hints of blocks and norms, see parts/base.py)
         order = [self.blocks[call.layer] for call in self.spec.schedule]

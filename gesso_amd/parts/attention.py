@@ -50,8 +50,23 @@ class Attention(Part):
         self.value_position = build("position", vp, rt) if vp is not None else None
         if self.value_position is not None and self.value_position.rotary_dim != self.value_dim:
             raise ValueError("values are turned over their whole width")
+        # a cap on the scores, kept first positions, a sink of the head's own: what only the general kernel knows
+        self.softcap = getattr(spec, "softcap", None)
+        self.keep_first = int(getattr(spec, "keep_first", 0) or 0)
+        self.head_sinks = bool(getattr(spec, "head_sinks", False))
+        self.capped = bool(self.softcap or self.keep_first or self.head_sinks)
+        self.plain_norm = spec.qk_norm is not None and not getattr(spec, "qk_norm_weight", True)
+        self.out_gate = getattr(spec, "out_gate", None)
+        if self.out_gate not in (None, "sigmoid", "silu"):
+            raise ValueError(f"the heads' gate is 'sigmoid' or 'silu', not {self.out_gate!r}")
+        self.value_mix = bool(getattr(spec, "value_mix", False))
+        if self.head_sinks and self.sink:
+            raise ValueError("the softmax's extra term is exp(0) or a head's own, not both")
+        if self.keep_first and not spec.window:
+            raise ValueError("kept first positions go with a window")
         self.plain = (self.value_dim == spec.head_dim and not self.chunk and not self.sink
-                      and self.value_position is None)
+                      and self.value_position is None and not self.capped and not self.plain_norm
+                      and self.out_gate is None and not self.value_mix)
 
     @staticmethod
     def tensor_specs(spec):
@@ -61,30 +76,47 @@ class Attention(Part):
                "v_proj.weight": TensorSpec((nkv * vd, H), MATRIX), "out_proj.weight": TensorSpec((H, nh * vd), MATRIX)}
         if spec.bias:
             out.update({"q_proj.bias": TensorSpec((nh * d,), VECTOR), "k_proj.bias": TensorSpec((nkv * d,), VECTOR),
-                        "v_proj.bias": TensorSpec((nkv * vd,), VECTOR), "out_proj.bias": TensorSpec((H,), VECTOR)})
-        if spec.qk_norm is not None:
+                        "v_proj.bias": TensorSpec((nkv * vd,), VECTOR)})
+        out_bias = getattr(spec, "out_bias", None)
+        if spec.bias if out_bias is None else out_bias:
+            out["out_proj.bias"] = TensorSpec((H,), VECTOR)
+        if spec.qk_norm is not None and getattr(spec, "qk_norm_weight", True):
             out.update({"q_norm.weight": TensorSpec((d,), VECTOR, "one_plus_normal"),
                         "k_norm.weight": TensorSpec((d,), VECTOR, "one_plus_normal")})
+        if getattr(spec, "head_sinks", False):
+            out["sinks"] = TensorSpec((nh,), VECTOR)
+        if getattr(spec, "out_gate", None) is not None:
+            out["gate_proj.weight"] = TensorSpec((nh * vd, H), MATRIX)
+        if getattr(spec, "value_mix", False):
+            out["value_mix"] = TensorSpec((), VECTOR)
         return out
 
     @staticmethod
     def cache_need(spec):
         vd = getattr(spec, "value_dim", None)
         return PagedKV(spec.n_kv_heads, spec.head_dim, spec.window, value_dim=None if vd in (None, spec.head_dim) else vd,
-                       chunk=getattr(spec, "chunk", None))
+                       chunk=getattr(spec, "chunk", None), keep_first=int(getattr(spec, "keep_first", 0) or 0))
 
     def bind(self, tensors):
         ws = [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]]
+        if self.out_gate is not None:
+            ws.append(tensors["gate_proj.weight"])       # the gate's product rides behind q | k | v
         if len({w.dtype for w in ws}) > 1:
             ws = [w.float() for w in ws]
         self.wqkv = self.rt.prepare(torch.cat(ws, 0).contiguous())
         self.wo = self.rt.prepare(tensors["out_proj.weight"])
-        self.bqkv = self.bo = None
+        self.bqkv = None
         if self.spec.bias:
-            self.bqkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]], 0).contiguous()
-            self.bo = tensors["out_proj.bias"]
+            bs = [tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]
+            if self.out_gate is not None:
+                bs.append(torch.zeros(ws[-1].shape[0], dtype=bs[0].dtype, device=bs[0].device))
+            self.bqkv = torch.cat(bs, 0).contiguous()
+        self.bo = tensors.get("out_proj.bias")
         self.q_norm = tensors.get("q_norm.weight")
         self.k_norm = tensors.get("k_norm.weight")
+        self.sinks = tensors.get("sinks")
+        mix = tensors.get("value_mix")
+        self.mix = None if mix is None else mix.reshape(1).contiguous()
 
     takes_out_dtype = True
 
@@ -92,6 +124,10 @@ class Attention(Part):
         q, q_stride = self.project_in(x, ctx, cache)
         with self.rt.stage("attn_core"):
             o = self.attend(q, q_stride, ctx, cache)
+            if self.out_gate is not None:
+                s = self.spec
+                o = self.rt.ops.gated_rows(self.rt.dense(o), q, (s.n_heads + s.n_kv_heads) * s.head_dim
+                                           + s.n_kv_heads * self.value_dim, self.out_gate)
         if out_dtype is not None:
             return self.rt.linear(o, self.wo, self.bo, out_dtype=out_dtype)
         return self.rt.project(o, self.wo, self.bo)
@@ -108,8 +144,17 @@ class Attention(Part):
         layout = getattr(pos, "layout", "half")
         with rt.stage("attn_proj"):
             qkv = rt.linear(x, self.wqkv, self.bqkv)      # a lazy norm goes through as it is where the product takes it
-        stride = (nh + nkv) * d + nkv * self.value_dim
+        stride = (nh + nkv) * d + nkv * self.value_dim + (nh * self.value_dim if self.out_gate is not None else 0)
         vp = self.value_position
+        v_first = mix = None
+        if self.value_mix:
+            # the first mixer of the step that shares its values keeps them (its rows stay as they are: only q is
+            # rewritten in place); the later ones blend theirs with them on the way into the cache
+            v_first = ctx.shared.get("value_mix")
+            if v_first is None:
+                ctx.shared["value_mix"] = qkv[:, (nh + nkv) * d:(nh + nkv) * d + nkv * self.value_dim]
+            else:
+                mix = self.mix
         if (self.plain and rt.fused and ctx.all_single and cache.k.dtype == torch.bfloat16 and qkv.dtype == torch.bfloat16
                 and cache.page_size >= 2 and (self.q_norm is None) == (self.k_norm is None) and layout == "half"
                 and ops.attention_decode_raw_supports(nh, nkv, d, pos.rotary_dim)):
@@ -118,7 +163,8 @@ class Attention(Part):
             ops.qknorm_rope_kv(qkv, self.q_norm, self.k_norm, eps, pos.cos, pos.sin, pos.rotary_dim, ctx.positions,
                                ctx.seq_of_token, cache.block_table, cache.page_size, cache.k, cache.v, nh, nkv, d,
                                write_kv=cache.write, layout=layout, vd=self.value_dim,
-                               vcos=None if vp is None else vp.cos, vsin=None if vp is None else vp.sin)
+                               vcos=None if vp is None else vp.cos, vsin=None if vp is None else vp.sin,
+                               plain_norm=self.plain_norm, v_first=v_first, mix=mix)
         return qkv, stride
 
     def _single(self, q, q_stride, cache, ctx, nseq, out):
@@ -213,6 +259,12 @@ class Attention(Part):
         s, rt, ops, vp = self.spec, self.rt, self.rt.ops, self.value_position
         layout = getattr(vp, "layout", "half") if vp is not None else "half"
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
+        if self.capped:
+            return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.block_table,
+                                         cache.page_size, s.window, self.scale, nh, nkv, d, ctx.T, vd=self.value_dim,
+                                         chunk=self.chunk, sink=self.sink, vcos=None if vp is None else vp.cos,
+                                         vsin=None if vp is None else vp.sin, layout=layout, softcap=self.softcap,
+                                         keep_first=self.keep_first, sinks=self.sinks)
         if (q.dtype == torch.bfloat16 and ctx.all_single and self.value_dim == d and cache.page_size >= 2
                 and q_stride % 8 == 0 and ops.attention_decode_supports(nh, nkv, d)):
             # single tokens whose values are as wide as their keys: the kernel for single queries, which knows runs and

@@ -53,6 +53,8 @@ class PagedKV:
     ``window``: only the last ``window`` tokens are ever read again (None = all of them).
     ``chunk``: positions are cut into runs of ``chunk`` from 0 on and a token reads only its own run, so the runs
     before the newest token's are never read again (None = no such cut).
+    ``keep_first``: the first positions of a sequence that stay readable when a window has passed them: the pages
+    that hold them are never given back while the request lives.
     """
 
     n_kv_heads: int
@@ -60,6 +62,11 @@ class PagedKV:
     window: Optional[int] = None
     value_dim: Optional[int] = None
     chunk: Optional[int] = None
+    keep_first: int = 0
+
+    def pages_kept(self, page_size: int) -> int:
+        """How many pages at a sequence's start hold positions that stay readable whatever has passed."""
+        return -(-int(self.keep_first) // page_size) if self.window is not None and self.chunk is None else 0
 
     def first_needed(self, length: int) -> int:
         """The oldest position that the token after ``length`` cached ones can read."""

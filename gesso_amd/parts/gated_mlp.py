@@ -56,4 +56,32 @@ class GatedMLP(Part):
         return rt.linear(a, self.w_down, self.b_down)
 
 
+class ClampedGLU(Part):
+    """``W_down (g sigmoid(alpha g) (u + 1))`` with ``g = min(W_gate x, limit)``, ``u = clamp(W_up x, -limit, limit)``:
+    the form a routed expert has (:mod:`gesso_amd.parts.routed_moe`), as a feed-forward of its own for every token."""
+
+    graph_safe = True
+    stage, out_stage = "dense_ffn", "ffn_down"
+
+    @staticmethod
+    def tensor_specs(spec):
+        H, F = spec.hidden, spec.intermediate
+        return {"gate.weight": TensorSpec((F, H), MATRIX), "up.weight": TensorSpec((F, H), MATRIX),
+                "down.weight": TensorSpec((H, F), MATRIX)}
+
+    def bind(self, tensors):
+        g, u = tensors["gate.weight"], tensors["up.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gu = self.rt.prepare(torch.cat([g, u], 0).contiguous(), unit=g.shape[0])
+        self.w_down = self.rt.prepare(tensors["down.weight"])
+
+    def forward(self, x, ctx):
+        rt, s = self.rt, self.spec
+        with rt.stage("ffn_gateup"):
+            a = rt.ops.clamped_glu(rt.linear(rt.dense(x), self.w_gu), s.limit, s.alpha, rt.dtype)
+        return rt.linear(a, self.w_down)
+
+
 register("ffn", "gated_mlp", GatedMLP)
+register("ffn", "clamped_glu", ClampedGLU)

@@ -10,7 +10,8 @@ type: activation, turn and scale are applied where the state kernel reads its op
 until norm and gate have been applied.
 
 ``MixerPair``: two mixers that read the same rows, each with a cache of its own; the result is
-``left_scale * left(x) + right_scale * right(x)``, summed in float32 and rounded once.
+``left_scale * left(x) + right_scale * right(x)``, summed in float32 and rounded once; with ``branch_norm_eps`` each side
+is first RMS-normed over the model width with a weight of its own.
 """
 from __future__ import annotations
 
@@ -110,6 +111,11 @@ class MixerPair(Part):
         for side, sub in (("left", spec.left), ("right", spec.right)):
             for name, ts in part_class("mixer", sub).tensor_specs(sub).items():
                 out[f"{side}.{name}"] = ts
+        if getattr(spec, "branch_norm_eps", None) is not None:
+            if spec.hidden is None:
+                raise ValueError("a pair that norms its branches must know the model width")
+            out["left_norm.weight"] = TensorSpec((spec.hidden,), VECTOR, "one_plus_normal")
+            out["right_norm.weight"] = TensorSpec((spec.hidden,), VECTOR, "one_plus_normal")
         return out
 
     @staticmethod
@@ -123,6 +129,7 @@ class MixerPair(Part):
     def bind(self, tensors):
         self.left.bind(sub_tensors(tensors, "left"))
         self.right.bind(sub_tensors(tensors, "right"))
+        self.left_norm, self.right_norm = tensors.get("left_norm.weight"), tensors.get("right_norm.weight")
 
     @property
     def graph_safe(self) -> bool:
@@ -136,6 +143,14 @@ class MixerPair(Part):
         kw = {"out_dtype": torch.float32} if wide else {}
         a = rt.dense(self.left.forward(x, ctx, cache[0], **kw))
         b = rt.dense(self.right.forward(x, ctx, cache[1], **kw))
+        eps = getattr(s, "branch_norm_eps", None)
+        if eps is not None:
+            # each side normed over the model width with its own weight, float32 from the products' sums to the one
+            # rounding of the weighted sum
+            if not wide:
+                a, b = a.float(), b.float()
+            return rt.ops.normed_pair_sum(a, self.left_norm, float(s.left_scale), b, self.right_norm, float(s.right_scale),
+                                          float(eps), rt.dtype)
         return rt.ops.scaled_sum(a, float(s.left_scale), b, float(s.right_scale), rt.dtype)
 
 

@@ -155,5 +155,36 @@ class GroupRMSNorm(Part):
         return y
 
 
+class LayerNorm(Part):
+    """``(x - mean) / sqrt(var + eps) * w + b`` over the last axis, the variance the mean of the squared deviations;
+    float32 arithmetic.  The pass adds what the sub-layer before left beside the stream, as the other norms' do."""
+
+    graph_safe = True
+
+    @staticmethod
+    def tensor_specs(spec):
+        out = {"weight": TensorSpec((spec.size,), VECTOR, "one_plus_normal")}
+        if getattr(spec, "bias", True):
+            out["bias"] = TensorSpec((spec.size,), VECTOR)
+        return out
+
+    def bind(self, tensors):
+        self.weight = tensors["weight"]
+        self.bias = tensors.get("bias")
+
+    def add_norm(self, stream: ResidualStream, rows=None, out=None, out_dtype=None):
+        """Add what is pending to the stream, then norm it (only ``rows`` of it when given)."""
+        rt = self.rt
+        if isinstance(stream.pending, tuple) or stream.bias is not None:
+            stream.flush(rt)
+        y = rt.ops.add_layernorm(stream.res, stream.pending, self.weight, self.bias, self.spec.eps, out_dtype or rt.dtype,
+                                 rows=rows, out=out)
+        if rows is None:
+            stream.pending = None
+        stream.ssq = stream.xs = stream.xs_for = stream.normed = stream.rows = None
+        return y
+
+
 register("norm", "rmsnorm", RMSNorm)
+register("norm", "layernorm", LayerNorm)
 register("norm", "group_rmsnorm", GroupRMSNorm)

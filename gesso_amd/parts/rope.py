@@ -16,9 +16,10 @@ from .base import Part
 from .registry import register
 
 
-def rope_tables(rotary_dim: int, theta: float, max_position: int):
+def rope_tables(rotary_dim: int, theta: float, max_position: int, divisor: float = 1.0):
+    """``divisor``: every frequency is divided by it (positions stretched evenly, "linear scaling")."""
     i = torch.arange(rotary_dim // 2, dtype=torch.float64)
-    inv_freq = torch.tensor(float(theta), dtype=torch.float64) ** (-2.0 * i / rotary_dim)
+    inv_freq = torch.tensor(float(theta), dtype=torch.float64) ** (-2.0 * i / rotary_dim) / float(divisor)
     ang = torch.arange(max_position, dtype=torch.float64)[:, None] * inv_freq[None, :]
     return torch.cos(ang).to(torch.float32), torch.sin(ang).to(torch.float32)
 
@@ -36,10 +37,11 @@ class Rope(Part):
             raise ValueError(f"rotation pairs are laid out 'half' or 'interleaved', not {self.layout!r}")
 
         def make():
-            cos, sin = rope_tables(spec.rotary_dim, spec.theta, spec.max_position)
+            cos, sin = rope_tables(spec.rotary_dim, spec.theta, spec.max_position, divisor)
             return cos.to(rt.device), sin.to(rt.device)
 
-        self.cos, self.sin = rt.shared(("rope", spec.rotary_dim, float(spec.theta), spec.max_position), make)
+        divisor = float(getattr(spec, "frequency_divisor", 1.0))
+        self.cos, self.sin = rt.shared(("rope", spec.rotary_dim, float(spec.theta), spec.max_position, divisor), make)
 
 
 def scaled_rope_tables(spec):

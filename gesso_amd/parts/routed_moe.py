@@ -1,7 +1,8 @@
 """A mixture of gated feed-forwards chosen by a router over the token's features.
 
-    z = W_r x  (float32),  s = softmax(z) over all ``E + I`` router outputs
+    z = W_r x  (float32),  s = softmax(z) over all ``E + I`` router outputs  (``score = "sigmoid"``: s = sigmoid(z))
     chosen: the ``top`` outputs with the largest ``s + correction``;  weights: ``s`` of the chosen / (their sum + 1e-20)
+    (``renormalize = False``: ``s`` of the chosen as they are), times ``route_scale``
     expert e < E:   W_down[e] (g sigmoid(alpha g) (u + 1)),  g = min(W_gate[e] x, limit),  u = clamp(W_up[e] x, -limit, limit)
     expert e >= E:  x itself (an identity expert: it has no tensors)
     y = sum over the chosen of weight * expert(x)  +  shared(x)   (an expert of its own width and limit, for every token)
@@ -61,7 +62,9 @@ class RoutedMoE(Part):
         s, rt, ops = self.spec, self.rt, self.rt.ops
         x = rt.dense(x)
         with rt.stage("ffn_router"):
-            choice, weight = ops.moe_router(x, self.router, self.correction, s.top)
+            choice, weight = ops.moe_router(x, self.router, self.correction, s.top, score=getattr(s, "score", "softmax"),
+                                            renormalize=getattr(s, "renormalize", True),
+                                            scale=getattr(s, "route_scale", 1.0))
         shared = None
         if self.w_sgu is not None:
             with rt.stage("ffn_shared"):
