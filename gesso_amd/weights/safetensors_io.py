@@ -126,7 +126,7 @@ def write_safetensors(path: str, tensors: Dict[str, torch.Tensor], metadata: Dic
         f.write(struct.pack("<Q", len(blob)))
         f.write(blob)
         for name, t in tensors.items():
-            c = t.detach().cpu().contiguous()
+            c = t.detach().cpu().contiguous().reshape(-1)       # (a tensor without axes has one value, too)
             if c.numel():
                 f.write(c.view(torch.uint8).numpy().tobytes() if c.dtype != torch.bool
                         else c.to(torch.uint8).numpy().tobytes())

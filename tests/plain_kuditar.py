@@ -48,6 +48,15 @@ ACTIVATION_SLOPE = 1.702
 UNIT_EPS = 1e-6
 
 
+def _keep(x):
+    return x
+
+
+def to_bfloat16(x: torch.Tensor) -> torch.Tensor:
+    """Round to bfloat16 and widen back: what a pipeline with bfloat16 activations does where it stores one."""
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
 def linear(x, W, b=None):
     y = x @ W.T
     return y if b is None else y + b
@@ -186,93 +195,94 @@ def _rot_freqs(m):
     return frequencies(int(rot["dims"]), float(rot["base"]), float(factor))
 
 
-def gated_attention(h, W, p, m, positions, eps, v_first=None):
-    """Mixer ``attention``.  Returns ``(output, this layer's own values)``."""
+def gated_attention(h, W, p, m, positions, eps, v_first=None, store=_keep):
+    """Mixer ``attention``.  Returns ``(output, this layer's own values)``.  ``store``: applied wherever a pipeline with
+    activations of another type would store one (here and in the functions below)."""
     T = h.shape[0]
     H, G, d, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = linear(h, W[p + "q"]).reshape(T, H, d)
-    k = linear(h, W[p + "k"]).reshape(T, G, d)
-    v = linear(h, W[p + "v"]).reshape(T, G, vd)
+    q = store(linear(h, W[p + "q"])).reshape(T, H, d)
+    k = store(linear(h, W[p + "k"])).reshape(T, G, d)
+    v = store(linear(h, W[p + "v"])).reshape(T, G, vd)
     f = _rot_freqs(m)
-    q, k = rms(rotate_half(q, positions, f), eps), rms(rotate_half(k, positions, f), eps)
+    q, k = store(rms(rotate_half(q, positions, f), eps)), store(rms(rotate_half(k, positions, f), eps))
     own = v
     if v_first is not None:
         lam = W[p + "vmix"]
-        v = (1 - lam) * v + lam * v_first
-    o = softmax_attention(q, k, v, positions, m["scale"], cap=m.get("softcap"))
-    o = o.reshape(T, H * vd) * torch.sigmoid(linear(h, W[p + "g"]))
-    return linear(o, W[p + "o"]), own
+        v = store((1 - lam) * v + lam * v_first)
+    o = store(softmax_attention(q, k, v, positions, m["scale"], cap=m.get("softcap")))
+    o = store(o.reshape(T, H * vd) * torch.sigmoid(store(linear(h, W[p + "g"]))))
+    return store(linear(o, W[p + "o"])), own
 
 
-def _normed_biased_heads(h, W, p, m, eps):
+def _normed_biased_heads(h, W, p, m, eps, store=_keep):
     T = h.shape[0]
     H, G, d, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = linear(h, W[p + "q"], W[p + "q.b"]).reshape(T, H, d)
-    k = linear(h, W[p + "k"], W[p + "k.b"]).reshape(T, G, d)
-    v = linear(h, W[p + "v"], W[p + "v.b"]).reshape(T, G, vd)
+    q = store(linear(h, W[p + "q"], W[p + "q.b"])).reshape(T, H, d)
+    k = store(linear(h, W[p + "k"], W[p + "k.b"])).reshape(T, G, d)
+    v = store(linear(h, W[p + "v"], W[p + "v.b"])).reshape(T, G, vd)
     return rms(q, eps) * W[p + "q.norm"], rms(k, eps) * W[p + "k.norm"], v
 
 
-def windowed_branch(h, W, p, m, positions, eps):
+def windowed_branch(h, W, p, m, positions, eps, store=_keep):
     """Left side of ``parallel``."""
-    q, k, v = _normed_biased_heads(h, W, p, m, eps)
+    q, k, v = _normed_biased_heads(h, W, p, m, eps, store)
     f = _rot_freqs(m)
-    q, k = rotate_half(q, positions, f), rotate_half(k, positions, f)
+    q, k = store(rotate_half(q, positions, f)), store(rotate_half(k, positions, f))
     mask = m.get("mask") or {}
     o = softmax_attention(q, k, v, positions, m["scale"], cap=m.get("softcap"), window=mask.get("size"),
                           keep_first=mask.get("keep_first") or 0, sink=W[p + "sink"])
-    return linear(o.reshape(h.shape[0], -1), W[p + "o"])
+    return linear(store(o).reshape(h.shape[0], -1), W[p + "o"])
 
 
-def chunked_branch(h, W, p, m, positions, eps):
+def chunked_branch(h, W, p, m, positions, eps, store=_keep):
     """Left side of ``parallel_2``."""
-    q, k, v = _normed_biased_heads(h, W, p, m, eps)
-    o = softmax_attention(q, k, v, positions, m["scale"], chunk=(m.get("mask") or {}).get("size"))
-    return linear(o.reshape(h.shape[0], -1), W[p + "o"])
+    q, k, v = _normed_biased_heads(h, W, p, m, eps, store)
+    o = softmax_attention(store(q), store(k), v, positions, m["scale"], chunk=(m.get("mask") or {}).get("size"))
+    return linear(store(o).reshape(h.shape[0], -1), W[p + "o"])
 
 
-def delta_branch(h, W, p, m, eps):
+def delta_branch(h, W, p, m, eps, store=_keep):
     """Right side of ``parallel``."""
     T = h.shape[0]
     H, G, n, vd = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = silu(causal_conv(linear(h, W[p + "q"]), W[p + "q.conv"])).reshape(T, G, n)
-    k = silu(causal_conv(linear(h, W[p + "k"]), W[p + "k.conv"])).reshape(T, G, n)
-    v = silu(causal_conv(linear(h, W[p + "v"]), W[p + "v.conv"])).reshape(T, H, vd)
+    q = silu(causal_conv(store(linear(h, W[p + "q"])), W[p + "q.conv"])).reshape(T, G, n)
+    k = silu(causal_conv(store(linear(h, W[p + "k"])), W[p + "k.conv"])).reshape(T, G, n)
+    v = silu(causal_conv(store(linear(h, W[p + "v"])), W[p + "v.conv"])).reshape(T, H, vd)
     q, k = unit(q) * n ** -0.5, unit(k)
-    beta = torch.sigmoid(linear(h, W[p + "b"]))
-    g = torch.exp(-torch.exp(W[p + "A_log"]) * softplus(linear(h, W[p + "a"]) + W[p + "dt_bias"]))
+    beta = torch.sigmoid(store(linear(h, W[p + "b"])))
+    g = torch.exp(-torch.exp(W[p + "A_log"]) * softplus(store(linear(h, W[p + "a"])) + W[p + "dt_bias"]))
     heads = []
     for hd in range(H):
         j = hd // (H // G)
         heads.append(rms(delta_rule(q[:, j], k[:, j], v[:, hd], beta[:, hd], g[:, hd]), eps) * W[p + "norm"])
-    o = torch.stack(heads, 1).reshape(T, H * vd) * silu(linear(h, W[p + "g"]))
+    o = store(torch.stack(heads, 1).reshape(T, H * vd) * silu(store(linear(h, W[p + "g"]))))
     return linear(o, W[p + "o"])
 
 
-def gated_linear_branch(h, W, p, m, eps):
+def gated_linear_branch(h, W, p, m, eps, store=_keep):
     """Right side of ``parallel_2``."""
     T = h.shape[0]
     H, n, vd = m["heads"], m["dim"], m["vdim"]
-    q = (linear(h, W[p + "q"]) * n ** -0.5).reshape(T, H, n)
-    k = linear(h, W[p + "k"]).reshape(T, H, n)
-    v = linear(h, W[p + "v"]).reshape(T, H, vd)
-    z = linear(linear(h, W[p + "a1"]), W[p + "a2"], W[p + "a2.b"])
+    q = (store(linear(h, W[p + "q"])) * n ** -0.5).reshape(T, H, n)
+    k = store(linear(h, W[p + "k"])).reshape(T, H, n)
+    v = store(linear(h, W[p + "v"])).reshape(T, H, vd)
+    z = linear(store(linear(h, W[p + "a1"])), W[p + "a2"], W[p + "a2.b"])
     alpha = (torch.sigmoid(z) ** (1.0 / m["tau"])).reshape(T, H, n)
     heads = [rms(gated_linear(q[:, hd], k[:, hd], v[:, hd], alpha[:, hd]), eps) * W[p + "norm"] for hd in range(H)]
-    o = torch.stack(heads, 1).reshape(T, H * vd) * silu(linear(h, W[p + "g"]))
+    o = store(torch.stack(heads, 1).reshape(T, H * vd) * silu(store(linear(h, W[p + "g"]))))
     return linear(o, W[p + "o"])
 
 
-def pair(left, right, W, p, eps):
-    return 0.5 * (rms(left, eps) * W[p + "left.out"] + rms(right, eps) * W[p + "right.out"])
+def pair(left, right, W, p, eps, store=_keep):
+    return store(0.5 * (rms(left, eps) * W[p + "left.out"] + rms(right, eps) * W[p + "right.out"]))
 
 
 # --------------------------------------------------------------------------- feed-forward
 
-def clamped_glu(h, W, p, limit):
-    g = torch.clamp(linear(h, W[p + "gate"]), max=limit)
-    u = torch.clamp(linear(h, W[p + "up"]), -limit, limit)
-    return linear(g * torch.sigmoid(ACTIVATION_SLOPE * g) * (u + 1), W[p + "down"])
+def clamped_glu(h, W, p, limit, store=_keep):
+    g = torch.clamp(store(linear(h, W[p + "gate"])), max=limit)
+    u = torch.clamp(store(linear(h, W[p + "up"])), -limit, limit)
+    return linear(store(g * torch.sigmoid(ACTIVATION_SLOPE * g) * (u + 1)), W[p + "down"])
 
 
 def route(h, W, p, top: int, scale: float):
@@ -283,67 +293,79 @@ def route(h, W, p, top: int, scale: float):
     return chosen, torch.gather(s, 1, chosen) * scale
 
 
-def moe(h, W, p, mlp):
+def moe(h, W, p, mlp, store=_keep):
     r = mlp["router"]
-    chosen, weights = route(h, W, p, r["top"], r["scale"])
+    chosen, weights = route(h, W, p, r["top"], r.get("scale") or 1.0)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(chosen[t].tolist(), weights[t]):
-            out[t] = out[t] + w * clamped_glu(h[t:t + 1], W, f"{p}e{e}.", mlp["expert"]["limit"])[0]
-    return out
+            out[t] = out[t] + w * clamped_glu(h[t:t + 1], W, f"{p}e{e}.", mlp["expert"]["limit"], store)[0]
+    return store(out)
 
 
-def feed_forward(h, W, p, mlp):
+def feed_forward(h, W, p, mlp, store=_keep):
     if mlp["kind"] == "dense":
-        return clamped_glu(h, W, p, mlp["limit"])
-    return moe(h, W, p, mlp)
+        return store(clamped_glu(h, W, p, mlp["limit"], store))
+    return moe(h, W, p, mlp, store)
 
 
 # --------------------------------------------------------------------------- the model
 
-def layer(x, W, i: int, entry, positions, eps, shared):
+def layer(x, W, i: int, entry, positions, eps, shared, store=_keep):
     """One layer on ``x (T, width)``; ``shared`` carries the first ``v_mix`` layer's values through the model."""
     p = f"l{i}."
     m = entry["mixer"]
-    h = layer_norm(x, W[p + "norm1"], W[p + "norm1.b"], eps)
+    h = store(layer_norm(x, W[p + "norm1"], W[p + "norm1.b"], eps))
     if entry["type"] == "attention":
         if m.get("v_mix"):
-            y, own = gated_attention(h, W, p + "mix.", m, positions, eps, shared.get("v_first"))
+            y, own = gated_attention(h, W, p + "mix.", m, positions, eps, shared.get("v_first"), store)
             shared.setdefault("v_first", own)
         else:
-            y, _ = gated_attention(h, W, p + "mix.", m, positions, eps)
+            y, _ = gated_attention(h, W, p + "mix.", m, positions, eps, None, store)
     elif entry["type"] == "parallel":
-        y = pair(windowed_branch(h, W, p + "mix.left.", m["left"], positions, eps),
-                 delta_branch(h, W, p + "mix.right.", m["right"], eps), W, p + "mix.", eps)
+        y = pair(windowed_branch(h, W, p + "mix.left.", m["left"], positions, eps, store),
+                 delta_branch(h, W, p + "mix.right.", m["right"], eps, store), W, p + "mix.", eps, store)
     elif entry["type"] == "parallel_2":
-        y = pair(chunked_branch(h, W, p + "mix.left.", m["left"], positions, eps),
-                 gated_linear_branch(h, W, p + "mix.right.", m["right"], eps), W, p + "mix.", eps)
+        y = pair(chunked_branch(h, W, p + "mix.left.", m["left"], positions, eps, store),
+                 gated_linear_branch(h, W, p + "mix.right.", m["right"], eps, store), W, p + "mix.", eps, store)
     else:
         raise ValueError(f"unknown layer type {entry['type']!r}")
     x = x + y
     if entry.get("mlp") is not None:
-        x = x + feed_forward(layer_norm(x, W[p + "norm2"], W[p + "norm2.b"], eps), W, p + "mlp.", entry["mlp"])
+        h = store(layer_norm(x, W[p + "norm2"], W[p + "norm2.b"], eps))
+        x = x + feed_forward(h, W, p + "mlp.", entry["mlp"], store)
     return x
 
 
-def forward(cfg: dict, W: dict, ids, dtype=torch.float64, streams=None):
-    """Logits ``(T, vocab)`` of one whole sequence from position 0.  ``streams``: a list that receives the stream after
-    every layer."""
-    W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in W.items()}
+def forward(cfg: dict, W: dict, ids, store=_keep, layers_out=None):
+    """Logits ``(T, vocab)`` of one whole sequence from position 0, in the tensors' type.  ``layers_out``: a list that
+    receives the stream after every layer."""
     eps = float(cfg["norm"]["eps"])
     positions = list(range(len(ids)))
     x = embedding(W["embed"], ids, float((cfg.get("embedding") or {}).get("scale") or 1.0))
     shared = {}
     for i, entry in enumerate(cfg["layers"]):
-        x = layer(x, W, i, entry, positions, eps, shared)
-        if streams is not None:
-            streams.append(x.clone())
-    return linear(layer_norm(x, W["final.norm"], W["final.norm.b"], eps), W["embed"])
+        x = layer(x, W, i, entry, positions, eps, shared, store)
+        if layers_out is not None:
+            layers_out.append(x.clone())
+    return linear(store(layer_norm(x, W["final.norm"], W["final.norm.b"], eps)), W["embed"])
 
 
-def load_folder(folder: str):
-    """``(config dictionary, tensors)`` of a model folder."""
+def greedy(cfg: dict, W: dict, prompt, n_new: int):
+    """The prompt and ``n_new`` tokens after it, each the largest logit's (the lowest id among equals), every step from
+    the whole sequence anew."""
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(torch.argmax(forward(cfg, W, ids)[-1])))
+    return ids
+
+
+def read_config(folder: str) -> dict:
+    with open(os.path.join(folder, "config.json"), encoding="utf-8") as f:
+        return json.load(f)
+
+
+def read_weights(folder: str, dtype=torch.float64) -> dict:
     from safetensors.torch import load_file
-    with open(os.path.join(folder, "config.json")) as f:
-        cfg = json.load(f)
-    return cfg, load_file(os.path.join(folder, "model.safetensors"))
+    return {k: (v.to(dtype) if v.is_floating_point() else v)
+            for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}

@@ -10,6 +10,7 @@ import numpy as np
 import torch
 
 import plain_fazezen
+import plain_kuditar
 import plain_lfm2
 import plain_makuzen
 import plain_togalorn
@@ -23,7 +24,7 @@ def plain_logits(model_dir: str, ids, rounded: bool = False) -> np.ndarray:
     rounded to bfloat16 wherever a pipeline with bfloat16 activations stores one."""
     # each architecture has its own plain implementation; all read a folder and offer forward(cfg, w, ids, store=)
     with open(os.path.join(model_dir, "config.json"), encoding="utf-8") as f:
-        P = {"Makuzen": plain_makuzen, "Fazezen": plain_fazezen, "Togalorn": plain_togalorn}.get(json.load(f).get("architecture"), plain_lfm2)
+        P = {"Makuzen": plain_makuzen, "Fazezen": plain_fazezen, "Togalorn": plain_togalorn, "Kuditar": plain_kuditar}.get(json.load(f).get("architecture"), plain_lfm2)
     cfg = P.read_config(model_dir)
     w = P.read_weights(model_dir, torch.float64)
     return P.forward(cfg, w, list(ids), **({"store": P.to_bfloat16} if rounded else {})).numpy()
