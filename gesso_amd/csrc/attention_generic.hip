@@ -60,14 +60,8 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
   for (int i = 0; i < GS_ATTN_MAX_D / 64; ++i) acc[i] = 0.f;
 
   // two runs of keys: the kept first positions lo0 .. hi0 - 1 (where there are any), then lo .. pos
-  const bool kept = hi0 > lo0;
-  for (int base = kept ? lo0 : lo, last = kept ? hi0 - 1 : pos; base <= pos;) {
-    if (base > last) {
-      if (last == pos) break;
-      base = lo;
-      last = pos;
-      continue;
-    }
+  for (int run = hi0 > lo0 ? 0 : 1; run < 2; ++run)
+  for (int base = run ? lo : lo0, last = run ? pos : hi0 - 1; base <= last; base += 64) {
     int u = base + lane;
     float s = -INFINITY;
     long off = 0;
@@ -99,7 +93,6 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, int q_stride, 
         acc[i] = a;
       }
     }
-    base += 64;
   }
   float inv = 1.0f / l;
   if (vcos) {

@@ -159,6 +159,9 @@ class Runtime:
         if (self.tile_weights and w.dtype == torch.bfloat16 and w.dim() == 2 and w.is_contiguous()
                 and w.shape[1] % 32 == 0 and unit % 16 == 0 and w.shape[0] % unit == 0):
             self._tiles[w.data_ptr()] = self.ops.tile_major(w)
+        else:
+            # (a weight bound earlier and freed since may have lain at this address: its copy is not this weight's)
+            self._tiles.pop(w.data_ptr(), None)
         return w
 
     def tiles_of(self, w):

@@ -246,6 +246,9 @@ def scan_case(ops, dtype, H, G, n, m, lens, cuts, per_channel, delta, seed=0, sl
             x[meet[0], junk + G * n + 1] = 6.0                      # one key along channel 1 ...
             x[meet[1], junk:junk + n] = 0.0
             x[meet[1], junk + 1] = 6.0                              # ... and, later, the query along the same channel
+        if delta:             # the delta rule is a contraction for keys no longer than one; longer keys make it grow without bound
+            kk = x[:, junk + G * n:junk + 2 * G * n].reshape(L, G, n)
+            x[:, junk + G * n:junk + 2 * G * n] = (kk / kk.norm(dim=-1, keepdim=True).clamp_min(1.0)).reshape(L, G * n)
         xs.append(x.to(dtype))
         decs.append(dec)
         betas.append(torch.rand(L, 2 + H, generator=g))
