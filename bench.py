@@ -498,6 +498,65 @@ def togalorn_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), 
     return out
 
 
+KUDITAR_SIZES = {
+    # eight layers: a pair with a window (attention beside the gated delta rule), gated attention that shares its values, a
+    # pair with runs (attention beside linear attention with channel decays), gated attention, and the same four again;
+    # the pairs' feed-forward is dense and as wide as Fazezen's, the attention layers' a mixture of experts as wide as
+    # Makuzen's; beside Fazezen of the same width and depth
+    "1024": dict(width=1024, attn=(16, 4, 64, 64), left=(16, 4, 64, 64), delta=(8, 4, 64, 128), decay=(8, 64, 128), window=512,
+                 run=512, ff=4608, experts=16, top=2, eff=512, vocab=65536, beside="1024"),
+    "2048": dict(width=2048, attn=(16, 4, 128, 128), left=(32, 8, 64, 64), delta=(16, 8, 64, 128), decay=(16, 64, 128), window=1024,
+                 run=1024, ff=8192, experts=32, top=4, eff=704, vocab=65536, beside="2048"),
+}
+
+
+def kuditar_config(size: str, max_position: int = 4096):
+    from gesso_amd.config import (ChannelDecayConfig, DeltaRuleConfig, DenseFFConfig, GatedAttentionConfig, KuditarConfig,
+                                  KuditarLayer, PairConfig, RunAttentionConfig, SigmoidMoEConfig, Turn, WindowedAttentionConfig)
+    z = KUDITAR_SIZES[size]
+    ah, ag, ad, avd = z["attn"]
+    lh, lg, ld, lvd = z["left"]
+    moe = SigmoidMoEConfig(z["experts"], z["top"], 2.5, z["eff"], 7.0)
+    dense = DenseFFConfig(z["ff"], 7.0)
+    attn = KuditarLayer("attention", GatedAttentionConfig(ah, ag, ad, avd, ad ** -0.5, 30.0, Turn(1e6, ad // 2, 8.0), True), moe)
+    windowed = KuditarLayer("parallel", PairConfig(
+        WindowedAttentionConfig(lh, lg, ld, lvd, ld ** -0.5, 30.0, Turn(1e6, ld), z["window"], 16), DeltaRuleConfig(*z["delta"], 4)), dense)
+    dh, dn, dm = z["decay"]
+    runs = KuditarLayer("parallel_2", PairConfig(RunAttentionConfig(lh, lg, ld, lvd, ld ** -0.5, None, None, z["run"]),
+                                                 ChannelDecayConfig(dh, dn, dm, 16.0, 16)), dense)
+    return KuditarConfig(vocab=z["vocab"], width=z["width"], layers=(windowed, attn, runs, attn) * 2, norm_eps=1e-6,
+                         embedding_scale=float(z["width"]) ** 0.5, max_position=max_position)
+
+
+def kuditar_workload(steps: int = 64, warmup: int = 8, sizes=("1024", "2048"), only: str = "", batches=(8, 64)) -> dict:
+    """Kuditar (pairs of softmax attention beside the gated delta rule or linear attention with channel decays, gated
+    attention with shared values, dense and routed feed-forwards behind layer norms) at two sets of layer sizes, beside
+    Fazezen of the same width and depth: a 2,048-token prompt in one step, and decode steps at 512-token prompts."""
+    from gesso_amd import Engine
+    from gesso_amd.parts import RuntimeOptions
+    out = {"metric": "Kuditar beside Fazezen at equal width and depth: prefill and decode tok/s", "unit": "tok/s", "dtype": "bf16",
+           "data": "synthetic: uniform random token ids, random weights N(0, 0.02)", "sizes": {}}
+    for size in sizes:
+        row = {}
+        for name, cfg in (("kuditar", kuditar_config(size)), ("fazezen", fazezen_config(KUDITAR_SIZES[size]["beside"]))):
+            if only and only != name:
+                continue
+            engine = Engine.from_config(cfg, seed=0, dtype="bfloat16", page_size=16, max_context=4096,
+                                        max_tokens=max(batches) * (512 + steps + warmup + 32) + 4096, num_slots=max(batches) + 1,
+                                        options=RuntimeOptions(tune_library=True))
+            sec = prefill_run(engine, cfg, 2048)
+            r = {"prefill_tok_s": round(2048 / sec, 1), "prefill_ms": round(sec * 1e3, 3), "weights_gb": round(weight_bytes(engine) / 1e9, 3)}
+            for b in batches:
+                dt, _ = decode_run(engine, cfg, b, 512, steps, warmup, seed=40 + b)
+                r[f"decode_b{b}_tok_s"] = round(b * steps / dt, 1)
+                r[f"decode_b{b}_ms"] = round(dt / steps * 1e3, 4)
+            row[name] = r
+            del engine
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -517,7 +576,7 @@ def main() -> int:
     ap.add_argument("--launched-portions", action="store_true", help="launch the steps with prompt portions kernel by kernel instead of "
                     "replaying recordings of them (the prefill of the default line, --workload serve)")
     ap.add_argument("--token-budget", type=int, default=4096, help="--workload serve: the most tokens a step holds")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen", "fazezen", "togalorn"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "long", "gemm", "stages", "makuzen", "fazezen", "togalorn", "kuditar"],
                     help="decode: the default line; serve: continuous batching at LFM2-350M sizes; long: LFM2-2.6B "
                          "sizes at a context of 32,768; gemm: the products of a 2,048-token prompt, ours beside the vendor's; "
                          "stages: the decode step stage by stage; makuzen: the Makuzen design at two sets of layer sizes "
@@ -526,6 +585,8 @@ def main() -> int:
     ap.add_argument("--fazezen-only", default="", choices=["", "fazezen", "lfm2"], help="--workload fazezen: one of the two models (for profiling)")
     ap.add_argument("--togalorn-sizes", default="1024,2048", help="--workload togalorn: which of its sizes")
     ap.add_argument("--togalorn-only", default="", choices=["", "togalorn", "makuzen"], help="--workload togalorn: one of the two models (for profiling)")
+    ap.add_argument("--kuditar-sizes", default="1024,2048", help="--workload kuditar: which of its sizes")
+    ap.add_argument("--kuditar-only", default="", choices=["", "kuditar", "fazezen"], help="--workload kuditar: one of the two models (for profiling)")
     ap.add_argument("--makuzen-sizes", default="1024,2048", help="--workload makuzen: which of its sizes")
     ap.add_argument("--makuzen-only", default="", choices=["", "makuzen", "lfm2"], help="--workload makuzen: one of the two models (for profiling)")
     args = ap.parse_args()
@@ -543,6 +604,10 @@ def main() -> int:
         if args.workload == "fazezen":
             print(json.dumps(fazezen_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.fazezen_sizes.split(",")),
                                               args.fazezen_only)))
+            return 0
+        if args.workload == "kuditar":
+            print(json.dumps(kuditar_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.kuditar_sizes.split(",")),
+                                              args.kuditar_only)))
             return 0
         if args.workload == "togalorn":
             print(json.dumps(togalorn_workload(min(args.steps, 64), min(args.warmup, 8), tuple(args.togalorn_sizes.split(",")),

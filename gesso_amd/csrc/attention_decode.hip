@@ -56,6 +56,12 @@ struct DecodeRaw {
   // positions; sink: one more term exp(0), without a value, in the softmax's denominator
   int chunk;
   int sink;
+  // softcap > 0: a score becomes softcap tanh(score / softcap).  keep_first > 0 (with a window, without runs): the
+  // sequence's first keep_first positions stay visible when the window has passed them.  sinks (one float32 a head):
+  // the extra term of the denominator is exp(sinks[h]) instead of exp(0).
+  float softcap;
+  int keep_first;
+  const float* sinks;
 };
 
 template <int D, int G, int W, int RAW>
@@ -82,8 +88,12 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
   const int pos = positions[seq];
-  int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
-  if (raw.chunk > 0 && pos - pos % raw.chunk > lo) lo = pos - pos % raw.chunk;
+  int lo_real = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  if (raw.chunk > 0 && pos - pos % raw.chunk > lo_real) lo_real = pos - pos % raw.chunk;
+  // The kept first positions that the window has passed stand before the window's keys in one row of places: place
+  // lo + i is key i for the `kept` first places, and key lo + i (itself) from there on.
+  const int kept = (raw.keep_first > 0 && window > 0 && raw.chunk == 0) ? (raw.keep_first < lo_real ? raw.keep_first : lo_real) : 0;
+  const int lo = lo_real - kept;
   const int nkeys = pos - lo + 1;
   // this block's share of the keys, in whole tiles of 64
   const int tiles = (nkeys + 63) >> 6;
@@ -96,6 +106,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
   // (u / page_size as one multiplication, page_magic = floor(2^32 / page_size) + 1, exact while u page_size < 2^32:
   // no branch near the loads, which would make the compiler wait for every load in flight)
   auto row_off = [&](int u) -> long {
+    u = u < lo_real ? u - lo : u;          // a place before the window's first key holds a kept first position
     const int pg = (int)__umulhi((unsigned)u, page_magic);
     const int r = u - pg * page_size;
     return (((long)bt[pg] * nkv + kvh) * page_size + r) * D;
@@ -294,7 +305,13 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool valid = base + 4 * (4 * kg + i) + kt <= pos;
-        sc[kt][i] = valid ? sc[kt][i] * qscale : -INFINITY;
+        float sv = sc[kt][i] * qscale;
+        if (raw.softcap > 0.f) {
+          // cap tanh(x / cap) = cap (1 - 2 / (1 + e^(2 x / cap))), in the base-2 units the scores are held in
+          const float e2 = __builtin_amdgcn_exp2f(sv * (2.f / raw.softcap));
+          sv = raw.softcap * DEC_LOG2E * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e2));
+        }
+        sc[kt][i] = valid ? sv : -INFINITY;
         mx = fmaxf(mx, sc[kt][i]);
       }
     const float mn = fmaxf(m, group4_max(mx));   // finite: a tile holds at least one key
@@ -404,7 +421,8 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
         }
     if (nsplit == 1) {
       // (a sink's score is 0; the maxima are in base-2 units of the scaled scores)
-      if (raw.sink) L += M > -INFINITY ? __builtin_amdgcn_exp2f(-M) : 1.f;
+      if (raw.sink || raw.sinks)
+        L += M > -INFINITY ? __builtin_amdgcn_exp2f((raw.sinks ? raw.sinks[kvh * G + g] * DEC_LOG2E : 0.f) - M) : 1.f;
       out[out_index(seq, (kvh * G + g) * D + j, nh * D, out_tiles)] = f32_to_bf16(o / L);
     } else {
       part_o[(unit * G + g) * D + j] = o;
@@ -422,7 +440,7 @@ __global__ __launch_bounds__(W * 64) void attention_decode_kernel(
 #define DEC_MAXSPLIT 64
 __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                               bf16* __restrict__ out, int nsplit, int nh, int nkv, int G, int D,
-                                              int out_tiles, int sink) {
+                                              int out_tiles, int sink, const float* __restrict__ sinks) {
   __shared__ float sm[DEC_MAXSPLIT][DEC_MAXG], sl[DEC_MAXSPLIT][DEC_MAXG], sf[DEC_MAXSPLIT][DEC_MAXG];
   __shared__ float sinv[DEC_MAXG];
   const int kvh = blockIdx.x, seq = blockIdx.y;
@@ -443,7 +461,7 @@ __global__ void attention_decode_merge_kernel(const float* __restrict__ part_o, 
       sf[sp][g] = f;
       L += sl[sp][g] * f;
     }
-    if (sink) L += M > -INFINITY ? __builtin_amdgcn_exp2f(-M) : 1.f;
+    if (sink || sinks) L += M > -INFINITY ? __builtin_amdgcn_exp2f((sinks ? sinks[kvh * G + g] * DEC_LOG2E : 0.f) - M) : 1.f;
     sinv[g] = 1.0f / L;
   }
   __syncthreads();
@@ -529,8 +547,11 @@ extern "C" long gs_attention_decode_workspace(int nseq, int nh, int nkv, int d, 
 static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache, const int* positions,
                         const int* block_table, int max_blocks, int page_size, int window, float scale, void* out,
                         int out_tiled, float* workspace, int nseq, int nh, int nkv, int d, int nsplit,
-                        const DecodeRaw* raw, hipStream_t stream, int chunk = 0, int sink = 0) {
+                        const DecodeRaw* raw, hipStream_t stream, int chunk = 0, int sink = 0, float softcap = 0.f,
+                        int keep_first = 0, const float* sinks = nullptr) {
   GS_REQUIRE(chunk >= 0, "attention_decode: bad chunk %d", chunk);
+  GS_REQUIRE(softcap >= 0.f && keep_first >= 0 && !(sink && sinks), "attention_decode: bad cap, kept positions or sinks");
+  GS_REQUIRE(keep_first == 0 || (window > 0 && chunk == 0), "attention_decode: kept first positions go with a window and no runs");
   GS_REQUIRE(!out_tiled || (nh * d) % 32 == 0, "attention_decode: tiled rows need a width that is a multiple of 32, not %d", nh * d);
   const int out_tiles = out_tiled ? gs_ceil_div(nseq, 16) : 0;
   GS_REQUIRE(gs_attention_decode_supports(nh, nkv, d), "attention_decode: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
@@ -553,9 +574,15 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   DecodeRaw none = {};
   none.chunk = chunk;
   none.sink = sink ? 1 : 0;
+  none.softcap = softcap;
+  none.keep_first = keep_first;
+  none.sinks = sinks;
   DecodeRaw with = raw ? *raw : none;
   with.chunk = chunk;
   with.sink = sink ? 1 : 0;
+  with.softcap = softcap;
+  with.keep_first = keep_first;
+  with.sinks = sinks;
 #define GS_ARGS                                                                                             \
   G, grid, stream, (const bf16*)q, q_stride, (bf16*)kcache, (bf16*)vcache, positions, block_table, max_blocks, \
       page_size, page_magic, window, scale, (bf16*)out, part_o, part_ml, nh, nkv, out_tiles
@@ -578,7 +605,7 @@ static int decode_entry(const void* q, int q_stride, void* kcache, void* vcache,
   if (nsplit > 1) {
     dim3 mgrid(nkv, nseq);
     attention_decode_merge_kernel<<<mgrid, 256, 0, stream>>>(part_o, part_ml, (bf16*)out, nsplit, nh, nkv, G, d, out_tiles,
-                                                             sink ? 1 : 0);
+                                                             sink ? 1 : 0, sinks);
     GS_LAUNCH_CHECK("attention_decode_merge");
   }
   return 0;
@@ -599,6 +626,17 @@ extern "C" int gs_attention_decode_runs(const void* q, int q_stride, const void*
                                         int nh, int nkv, int d, int nsplit, int chunk, int sink, hipStream_t stream) {
   return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
                       scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream, chunk, sink);
+}
+
+// The same with a cap on the scores, kept first positions and sinks of the heads' own as well (see DecodeRaw).
+extern "C" int gs_attention_decode_rules(const void* q, int q_stride, const void* kcache, const void* vcache,
+                                         const int* positions, const int* block_table, int max_blocks, int page_size,
+                                         int window, float scale, void* out, int out_tiled, float* workspace, int nseq,
+                                         int nh, int nkv, int d, int nsplit, int chunk, int sink, float softcap,
+                                         int keep_first, const float* sinks, hipStream_t stream) {
+  return decode_entry(q, q_stride, (void*)kcache, (void*)vcache, positions, block_table, max_blocks, page_size, window,
+                      scale, out, out_tiled, workspace, nseq, nh, nkv, d, nsplit, nullptr, stream, chunk, sink, softcap,
+                      keep_first, sinks);
 }
 
 // ---- the entry point that allocates nothing (declared and described in no_alloc.h)

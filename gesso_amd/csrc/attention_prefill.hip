@@ -14,8 +14,11 @@ extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kca
                                     const int* positions, const int* tile_seq, const int* tile_row,
                                     const int* tile_n, int ntiles, const int* block_table, int max_blocks,
                                     int page_size, int window, float scale, void* out, int nh, int nkv, int d,
-                                    int tile_rows, int chunk, int sink, hipStream_t stream) {
+                                    int tile_rows, int chunk, int sink, float softcap, int keep_first,
+                                    const float* sinks, hipStream_t stream) {
   GS_REQUIRE(chunk >= 0, "attention_prefill: bad chunk %d", chunk);
+  GS_REQUIRE(softcap >= 0.f && keep_first >= 0 && !(sink && sinks), "attention_prefill: bad cap, kept positions or sinks");
+  GS_REQUIRE(keep_first == 0 || (window > 0 && chunk == 0), "attention_prefill: kept first positions go with a window and no runs");
   GS_REQUIRE(gs_attention_prefill_supports(nh, nkv, d), "attention_prefill: sizes nh=%d nkv=%d d=%d are not taken", nh, nkv, d);
   GS_REQUIRE(ntiles >= 0 && nkv > 0 && (long)ntiles * nkv < (1L << 31), "attention_prefill: %d tiles x %d key heads are too many blocks", ntiles, nkv);
   GS_REQUIRE(tile_rows == 16 || tile_rows == 32, "attention_prefill: tiles hold 16 or 32 queries, not %d", tile_rows);
@@ -30,7 +33,7 @@ extern "C" int gs_attention_prefill(const void* q, int q_stride, const void* kca
   const unsigned page_magic = (unsigned)((1ull << 32) / (unsigned)page_size + 1);
   PrefillCall c = {(const bf16*)q, (const bf16*)kcache, (const bf16*)vcache, positions, tile_seq, tile_row, tile_n,
                    block_table, q_stride, max_blocks, page_size, window, nh, nkv, tile_rows, ntiles, chunk, sink ? 1 : 0,
-                   page_magic, scale, (bf16*)out, stream};
+                   keep_first, page_magic, scale, softcap, sinks, (bf16*)out, stream};
   int rc = -1;
   switch (d) {
     case 32: rc = gs_attention_prefill_d32(c); break;

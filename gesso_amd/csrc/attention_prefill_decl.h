@@ -6,9 +6,10 @@ struct PrefillCall {
   const bf16 *q, *kc, *vc;
   const int *positions, *tile_seq, *tile_row, *tile_n, *bt;
   int q_stride, max_blocks, page_size, window, nh, nkv, tile_rows, ntiles;
-  int chunk, sink;
+  int chunk, sink, keep_first;
   unsigned page_magic;
-  float scale;
+  float scale, softcap;
+  const float* sinks;
   bf16* out;
   hipStream_t stream;
 };

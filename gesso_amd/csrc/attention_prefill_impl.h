@@ -16,7 +16,11 @@
 //
 // Causal rule: the query at position p sees keys lo..p, lo = 0 or p - window + 1; with chunk > 0 no further back
 // than the first position of p's own run of `chunk` positions.  With `sink` the softmax's denominator has one more
-// term, exp(0), which has no value.  Tiles of queries come
+// term, exp(0), which has no value; with `sinks` (one float32 a head) that term is exp(sinks[h]).  softcap > 0: a score
+// becomes softcap tanh(score / softcap) (the tanh from one exponential and one reciprocal).  keep_first > 0 (with a
+// window, without runs): the sequence's first keep_first positions stay visible when the window has passed them; the
+// tile walks those of them that lie before its window's first key in a walk of their own, ahead of the window's.
+// Tiles of queries come
 // from the host: tile i covers rows tile_row[i] .. + tile_n[i] (at most 16 QT) of the flattened tokens, of
 // sequence tile_seq[i].  Exponentials are base 2 on scores scaled by log2(e): one v_exp_f32 each.  q (T, q_stride), head h at [h D, (h+1) D); caches (pages, nkv, page_size, D); out (T, nh D).
 #pragma once
@@ -41,7 +45,8 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
     const bf16* __restrict__ q, int q_stride, const bf16* __restrict__ kcache, const bf16* __restrict__ vcache,
     const int* __restrict__ positions, const int* __restrict__ tile_seq, const int* __restrict__ tile_row,
     const int* __restrict__ tile_n, const int* __restrict__ block_table, int max_blocks, int page_size,
-    unsigned page_magic, int window, float scale, bf16* __restrict__ out, int nh, int nkv, int chunk, int sink) {
+    unsigned page_magic, int window, float scale, bf16* __restrict__ out, int nh, int nkv, int chunk, int sink,
+    float softcap, int keep_first, const float* __restrict__ sinks) {
   constexpr int PF_KSTEP = D <= 64 ? 64 : 32;   // keys per step: what three sets of row registers allow
   constexpr int KK = D / 32;   // feature steps of the score product
   constexpr int DT = D / 16;   // feature tiles of the output
@@ -70,7 +75,10 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   };
   const int first_key = lo_of(pos0);
   // scores are kept in units of log2(e), so that the exponentials are single v_exp_f32
-  const float sc = scale * PF_LOG2E;
+  // (capped scores are brought to those units where they are capped, and are scaled no more)
+  const bool capped = softcap > 0.f;
+  const float sc = capped ? 1.f : scale * PF_LOG2E;
+  const float cap_in = capped ? 2.f * PF_LOG2E * scale / softcap : 0.f, cap_out = softcap * PF_LOG2E;
 
   bool live[QT];
   int my_pos[QT], my_lo[QT];
@@ -100,9 +108,7 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   // around a load makes the compiler wait for every load in flight).  The LDS copy holds PF_MAXPAGES pages; a
   // longer key range is walked window by window.  u / page_size is a multiplication: page_magic =
   // floor(2^32 / page_size) + 1 is exact for u page_size < 2^32.
-  const int blk0 = (int)__umulhi((unsigned)first_key, page_magic);
-  const int blk1 = (int)__umulhi((unsigned)last_key, page_magic);
-  int win_blk = blk0, win_first = first_key, win_last = last_key;   // the window's pages and keys
+  int win_blk = 0, win_first = first_key, win_last = last_key;   // the window's pages and keys
   // Rows outside the window's keys are never seen (their scores are masked): their addresses are clamped
   // into the range, so that every load is of a row the sequence holds and no load needs a branch.
   auto row_of = [&](int u, bool clamp) -> size_t {
@@ -138,12 +144,14 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
     else fetch_as(stage, std::false_type{}, k0);
   };
   // per query: the last key it sees and the first, relative to this lane's rows of a score tile (4 kg + i)
-  int hi[QT], lo[QT];
+  int hi[QT], lo[QT], lo_own[QT];
 #pragma unroll
   for (int t = 0; t < QT; ++t) {
     hi[t] = live[t] ? my_pos[t] - kg * 4 : -(1 << 30);
-    lo[t] = my_lo[t] - kg * 4;
+    lo[t] = lo_own[t] = my_lo[t] - kg * 4;
   }
+  // keys below `keepk` (in this lane's rows) are kept first positions: seen whatever the window says
+  const int keepk = (keep_first > 0 ? keep_first : -(1 << 30)) - kg * 4;
 
   // A step whose keys every query of the tile sees (`inner`: below the diagonal, inside the windows) needs no
   // masks; most steps are such, and the masks are a third of a step's instructions.
@@ -183,8 +191,14 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int key = k0 + b * 16 + i;           // + 4 kg, which hi and lo already hold
-          if (MASK) s[t][b * 4 + i] = (key <= hi[t] && key >= lo[t] && key <= whi && key >= wlo) ? st[t][i] : -INFINITY;
-          else s[t][b * 4 + i] = st[t][i];
+          float sv = st[t][i];
+          if (capped) {
+            // cap tanh(x / cap) = cap (1 - 2 / (1 + e^(2 x / cap))), in units of log2(e)
+            const float e2 = __builtin_amdgcn_exp2f(sv * cap_in);
+            sv = cap_out * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e2));
+          }
+          if (MASK) s[t][b * 4 + i] = (key <= hi[t] && (key >= lo[t] || key < keepk) && key <= whi && key >= wlo) ? sv : -INFINITY;
+          else s[t][b * 4 + i] = sv;
         }
     }
     bf16x8_t pf[QT][NB / 2];
@@ -235,33 +249,49 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   };
   const int last_lo = lo_of(last_key);
   auto step = [&](auto stage, int k0) {
+    // (in the walk over kept first positions win_last lies before last_lo, so no step of it is taken for inner)
     const bool inner = k0 + PF_KSTEP - 1 <= pos0 && k0 >= last_lo && k0 >= win_first && k0 + PF_KSTEP - 1 <= win_last &&
                        nq == 16 * QT;
     if (inner) step_as(stage, std::true_type{}, k0);
     else step_as(stage, std::false_type{}, k0);
   };
 
-  for (win_blk = blk0; win_blk <= blk1; win_blk += PF_MAXPAGES) {
-    const int wend = win_blk + PF_MAXPAGES - 1 < blk1 ? win_blk + PF_MAXPAGES - 1 : blk1;
-    __syncthreads();                 // nobody reads the previous window any more
-    for (int i = tid; i <= wend - win_blk; i += GT * KSPLIT) pages[i] = bt[win_blk + i];
-    __syncthreads();
-    win_first = win_blk * page_size > first_key ? win_blk * page_size : first_key;
-    win_last = (wend + 1) * page_size - 1 < last_key ? (wend + 1) * page_size - 1 : last_key;
-    // the sets take the steps in turn; all make the same number of steps (the barriers are the block's), a set
-    // whose step lies beyond the keys computes on masked scores
-    const int kstart = (win_first / PF_KSTEP) * PF_KSTEP + grp * PF_KSTEP;
-    constexpr int STRIDE = KSPLIT * PF_KSTEP;
-    fetch(std::integral_constant<int, 0>{}, kstart);
-    fetch(std::integral_constant<int, 1>{}, kstart + STRIDE);
-    for (int k0 = kstart; k0 - grp * PF_KSTEP <= win_last; k0 += 3 * STRIDE) {
-      step(std::integral_constant<int, 0>{}, k0);
-      if (k0 - grp * PF_KSTEP + STRIDE > win_last) break;
-      step(std::integral_constant<int, 1>{}, k0 + STRIDE);
-      if (k0 - grp * PF_KSTEP + 2 * STRIDE > win_last) break;
-      step(std::integral_constant<int, 2>{}, k0 + 2 * STRIDE);
+  // One walk over the keys range_first .. range_last: by windows of pages, the sets of wavefronts taking the steps in turn.
+  auto walk = [&](int range_first, int range_last) {
+    const int b0 = (int)__umulhi((unsigned)range_first, page_magic), b1 = (int)__umulhi((unsigned)range_last, page_magic);
+    for (win_blk = b0; win_blk <= b1; win_blk += PF_MAXPAGES) {
+      const int wend = win_blk + PF_MAXPAGES - 1 < b1 ? win_blk + PF_MAXPAGES - 1 : b1;
+      __syncthreads();                 // nobody reads the previous window any more
+      for (int i = tid; i <= wend - win_blk; i += GT * KSPLIT) pages[i] = bt[win_blk + i];
+      __syncthreads();
+      win_first = win_blk * page_size > range_first ? win_blk * page_size : range_first;
+      win_last = (wend + 1) * page_size - 1 < range_last ? (wend + 1) * page_size - 1 : range_last;
+      // the sets take the steps in turn; all make the same number of steps (the barriers are the block's), a set
+      // whose step lies beyond the keys computes on masked scores
+      const int kstart = (win_first / PF_KSTEP) * PF_KSTEP + grp * PF_KSTEP;
+      constexpr int STRIDE = KSPLIT * PF_KSTEP;
+      fetch(std::integral_constant<int, 0>{}, kstart);
+      fetch(std::integral_constant<int, 1>{}, kstart + STRIDE);
+      for (int k0 = kstart; k0 - grp * PF_KSTEP <= win_last; k0 += 3 * STRIDE) {
+        step(std::integral_constant<int, 0>{}, k0);
+        if (k0 - grp * PF_KSTEP + STRIDE > win_last) break;
+        step(std::integral_constant<int, 1>{}, k0 + STRIDE);
+        if (k0 - grp * PF_KSTEP + 2 * STRIDE > win_last) break;
+        step(std::integral_constant<int, 2>{}, k0 + 2 * STRIDE);
+      }
     }
+  };
+  // the kept first positions that lie before the first key of the tile's window: a walk of their own, in which no
+  // query's window counts (every one of these keys is before every query's window, and all of them are kept)
+  const int kept_end = (keep_first > 0 && window > 0) ? (keep_first < first_key ? keep_first : first_key) : 0;
+  if (kept_end > 0) {
+#pragma unroll
+    for (int t = 0; t < QT; ++t) lo[t] = -(1 << 30);
+    walk(0, kept_end - 1);
+#pragma unroll
+    for (int t = 0; t < QT; ++t) lo[t] = lo_own[t];
   }
+  walk(first_key, last_key);
   if (KSPLIT > 1) {
     // add up the sets, in set order: set 0 takes the others' (reference point, sum, accumulator) through LDS,
     // one tile of queries at a time
@@ -304,7 +334,8 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
   for (int t = 0; t < QT; ++t) {
     if (!live[t]) continue;
     // a sink: one more term in the denominator, of score 0 (scores are held relative to m, in units of log2 e)
-    if (sink) l[t] += m[t] == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(-m[t]);
+    // (a head's own sink has the score sinks[h], unscaled and uncapped)
+    if (sink || sinks) l[t] += m[t] == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((sinks ? sinks[h] * PF_LOG2E : 0.f) - m[t]);
     const float inv = 1.0f / l[t];
     bf16* orow = out + (size_t)(row0 + t * 16 + r16) * nh * D + (size_t)h * D;
 #pragma unroll
@@ -321,12 +352,13 @@ template <int D, int QT, int KSPLIT>
 static int launch_prefill(int G, dim3 grid, hipStream_t stream, const bf16* q, int q_stride, const bf16* kc,
                           const bf16* vc, const int* positions, const int* tile_seq, const int* tile_row,
                           const int* tile_n, const int* bt, int max_blocks, int page_size, unsigned page_magic,
-                          int window, float scale, bf16* out, int nh, int nkv, int chunk, int sink) {
+                          int window, float scale, bf16* out, int nh, int nkv, int chunk, int sink, float softcap,
+                          int keep_first, const float* sinks) {
 #define GS_RUN(GG)                                                                                                   \
   if constexpr (KSPLIT > 1 && GG > 4) return -1;                                                                        \
   else attention_prefill_kernel<D, GG, QT, KSPLIT><<<grid, GG * KSPLIT * 64, 0, stream>>>(q, q_stride, kc, vc, positions, tile_seq, tile_row, \
                                                                 tile_n, bt, max_blocks, page_size, page_magic, window, \
-                                                                scale, out, nh, nkv, chunk, sink)
+                                                                scale, out, nh, nkv, chunk, sink, softcap, keep_first, sinks)
   switch (G) {
     case 1: GS_RUN(1); break;
     case 2: GS_RUN(2); break;
@@ -353,7 +385,7 @@ static int prefill_for_width(const PrefillCall& c) {
   const bool split = G <= 4;
 #define GS_ARGS                                                                                                    \
   G, grid, c.stream, c.q, c.q_stride, c.kc, c.vc, c.positions, c.tile_seq, c.tile_row, c.tile_n, c.bt, c.max_blocks, \
-      c.page_size, c.page_magic, c.window, c.scale, c.out, c.nh, c.nkv, c.chunk, c.sink
+      c.page_size, c.page_magic, c.window, c.scale, c.out, c.nh, c.nkv, c.chunk, c.sink, c.softcap, c.keep_first, c.sinks
   if (c.tile_rows == 16) return split ? launch_prefill<D, 1, 2>(GS_ARGS) : launch_prefill<D, 1, 1>(GS_ARGS);
   return split ? launch_prefill<D, 2, 2>(GS_ARGS) : launch_prefill<D, 2, 1>(GS_ARGS);
 #undef GS_ARGS

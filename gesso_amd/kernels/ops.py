@@ -925,11 +925,15 @@ def _decode_workspace(device, nseq, nh, nkv, d, nsplit):
 
 
 def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_size, window, scale, nh, nkv, d, nseq,
-                     nsplit: int, out=None, chunk: int = None, sink: bool = False):
+                     nsplit: int, out=None, chunk: int = None, sink: bool = False, softcap: float = None,
+                     keep_first: int = 0, sinks=None):
     """One query per sequence over its paged keys (bfloat16), keys split over ``nsplit`` blocks per key head.
     ``out``: a tensor, or True / a :class:`TiledRows` for tiled rows.  ``chunk``: the query sees only the keys of its
-    own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator."""
-    _dev(q, kcache, vcache, positions, block_table, out if isinstance(out, torch.Tensor) else None)
+    own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator; ``softcap``: scores
+    become ``softcap tanh(score / softcap)``; ``keep_first``: with a window, the sequence's first positions that stay
+    visible beyond it; ``sinks (nh,)`` float32: the extra term is ``exp(sinks[h])``."""
+    _dev(q, kcache, vcache, positions, block_table, out if isinstance(out, torch.Tensor) else None, sinks)
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (nh,)), "attention_decode: sinks must be float32 (nh,)")
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_decode takes bfloat16")
     _need(q.numel() >= (nseq - 1) * q_stride + nh * d if nseq else True, "attention_decode: q is too small")
@@ -941,6 +945,14 @@ def attention_decode(q, q_stride, kcache, vcache, positions, block_table, page_s
     ws = _decode_workspace(q.device, nseq, nh, nkv, d, nsplit)
     out, buf, tiled = _rows_out(out, nseq, nh * d, q.device, q.dtype)
     _need(tuple(out.shape) == (nseq, nh * d) and out.dtype == q.dtype, "attention_decode: out has the wrong shape or type")
+    if softcap or keep_first or sinks is not None:
+        _check(lib().gs_attention_decode_rules(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
+                                               c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0),
+                                               c_float(scale), _p(buf), c_int(tiled), _p(ws), c_int(nseq), c_int(nh),
+                                               c_int(nkv), c_int(d), c_int(nsplit), c_int(chunk or 0),
+                                               c_int(1 if sink else 0), c_float(softcap or 0.0), c_int(keep_first or 0),
+                                               _p(sinks), _stream()))
+        return out
     if chunk or sink:
         _check(lib().gs_attention_decode_runs(_p(q), c_int(q_stride), _p(kcache), _p(vcache), _p(positions), _p(block_table),
                                               c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0),
@@ -1010,14 +1022,18 @@ def turn_heads(x, cos, sin, positions, nh: int, w: int, sign: float = 1.0, layou
 
 
 def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table, page_size, window, scale, nh, nkv, d,
-                      ntok, out: torch.Tensor = None, tile_rows: int = 16, chunk: int = None, sink: bool = False) -> torch.Tensor:
+                      ntok, out: torch.Tensor = None, tile_rows: int = 16, chunk: int = None, sink: bool = False,
+                      softcap: float = None, keep_first: int = 0, sinks=None) -> torch.Tensor:
     """Causal GQA of many queries per sequence on the matrix cores (bfloat16).  ``chunk``: a query sees only the keys
-    of its own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator.
+    of its own run of ``chunk`` positions; ``sink``: one more term ``exp(0)`` in the softmax's denominator;
+    ``softcap``: scores become ``softcap tanh(score / softcap)``; ``keep_first``: with a window, the sequence's first
+    positions that stay visible beyond it; ``sinks (nh,)`` float32: the extra term is ``exp(sinks[h])``.
 
     ``tiles``: int32 ``(3, ntiles)``: sequence, first row and number of rows (at most ``tile_rows``, 16 or
     32) of each tile of consecutive queries of one sequence.
     """
-    _dev(q, kcache, vcache, positions, tiles, block_table, out)
+    _dev(q, kcache, vcache, positions, tiles, block_table, out, sinks)
+    _need(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (nh,)), "attention_prefill: sinks must be float32 (nh,)")
     _need(q.dtype == torch.bfloat16 and kcache.dtype == torch.bfloat16 and vcache.dtype == torch.bfloat16,
           "attention_prefill takes bfloat16")
     _need(q.numel() >= (ntok - 1) * q_stride + nh * d if ntok else True, "attention_prefill: q is too small")
@@ -1034,7 +1050,8 @@ def attention_prefill(q, q_stride, kcache, vcache, positions, tiles, block_table
                                       _p(tiles[1]), _p(tiles[2]), c_int(nt), _p(block_table),
                                       c_int(block_table.shape[1]), c_int(page_size), c_int(window or 0), c_float(scale),
                                       _p(out), c_int(nh), c_int(nkv), c_int(d), c_int(tile_rows), c_int(chunk or 0),
-                                      c_int(1 if sink else 0), _stream()))
+                                      c_int(1 if sink else 0), c_float(softcap or 0.0), c_int(keep_first or 0), _p(sinks),
+                                      _stream()))
     return out
 
 

@@ -260,6 +260,31 @@ class Attention(Part):
         layout = getattr(vp, "layout", "half") if vp is not None else "half"
         nh, nkv, d = s.n_heads, s.n_kv_heads, s.head_dim
         if self.capped:
+            if (q.dtype == torch.bfloat16 and ctx.all_single and self.value_dim == d and cache.page_size >= 2
+                    and q_stride % 8 == 0 and ops.attention_decode_supports(nh, nkv, d) and vp is None
+                    and not (self.keep_first and self.chunk)):
+                # single tokens whose values are as wide as their keys: the kernel for single queries, which knows the
+                # cap, the kept first positions (they stand before the window's keys in its row of places) and the sinks
+                longest = ctx.max_kv_len if ctx.max_kv_len is not None else cache.block_table.shape[1] * cache.page_size
+                if s.window:
+                    longest = min(longest, s.window + self.keep_first)
+                if self.chunk:
+                    longest = min(longest, self.chunk)
+                tiles = max(1, -(-longest // 64))
+                nsplit = max(1, min(tiles // 16, 64, 256 // max(1, ctx.nseq * nkv)))
+                return ops.attention_decode(q, q_stride, cache.k, cache.v, ctx.positions, cache.block_table, cache.page_size,
+                                            s.window, self.scale, nh, nkv, d, ctx.nseq, nsplit, chunk=self.chunk, sink=self.sink,
+                                            softcap=self.softcap, keep_first=self.keep_first, sinks=self.sinks)
+            if (q.dtype == torch.bfloat16 and not ctx.all_single and self.value_dim == d and cache.page_size >= 2
+                    and q_stride % 8 == 0 and ops.attention_prefill_supports(nh, nkv, d) and ctx.recording is None
+                    and vp is None and not (self.keep_first and self.chunk)):
+                # prompt portions whose values are as wide as their keys: the kernel on the matrix cores, which knows
+                # the cap, the kept first positions and the heads' own sinks
+                rows = 32 if ctx.max_q_len >= 64 and nh // nkv <= 4 else 16
+                return ops.attention_prefill(q, q_stride, cache.k, cache.v, ctx.positions, ctx.query_tiles(rows, 0),
+                                             cache.block_table, cache.page_size, s.window, self.scale, nh, nkv, d, ctx.T,
+                                             tile_rows=rows, chunk=self.chunk, sink=self.sink, softcap=self.softcap,
+                                             keep_first=self.keep_first, sinks=self.sinks)
             return ops.attention_generic(q, q_stride, cache.k, cache.v, ctx.positions, ctx.seq_of_token, cache.block_table,
                                          cache.page_size, s.window, self.scale, nh, nkv, d, ctx.T, vd=self.value_dim,
                                          chunk=self.chunk, sink=self.sink, vcos=None if vp is None else vp.cos,

@@ -115,12 +115,24 @@ class Pages:
         self.ps = page_size
 
 
+def tiles_of(sizes, rows):
+    """int32 ``(3, ntiles)``: sequence, first row and row count of tiles of at most ``rows`` queries of one sequence."""
+    seq, row, cnt, at = [], [], [], 0
+    for i, n in enumerate(sizes):
+        for a in range(0, n, rows):
+            seq.append(i)
+            row.append(at + a)
+            cnt.append(min(rows, n - a))
+        at += n
+    return i32([seq, row, cnt])
+
+
 def attention_case(ops, dtype, nh, nkv, d, vd, lens, cuts, ps=8, window=None, keep_first=0, chunk=None, cap=None, sinks=None,
-                   scale=0.3, seed=0, plant=None):
+                   scale=0.3, seed=0, plant=None, tiled=0):
     """Sequences of ``lens`` tokens fed in the pieces ``cuts[s]``: raw q | k | v rows go through the cache write (no norm,
     no turn) and the general attention kernel.  ``plant``: ``(sequence, key position, query position, size)``: that key is
-    made to point along that query's first head, ``size`` times as long.  Returns the kernel's rows and the plain
-    attention's, per sequence."""
+    made to point along that query's first head, ``size`` times as long.  ``tiled``: 16 or 32: the kernel on the matrix
+    cores with tiles of that many queries instead.  Returns the kernel's rows and the plain attention's, per sequence."""
     g = gen(seed)
     rows = [torch.randn(n, (nh + nkv) * d + nkv * vd, generator=g) for n in lens]
     if plant is not None:
@@ -140,8 +152,17 @@ def attention_case(ops, dtype, nh, nkv, d, vd, lens, cuts, ps=8, window=None, ke
         seq_of = [i for i, n in enumerate(sizes) for _ in range(n)]
         table = pg.table[live].contiguous()
         ops.qknorm_rope_kv(x, None, None, 1.0, None, None, 0, i32(pos), i32(seq_of), table, ps, pg.k, pg.v, nh, nkv, d, vd=vd)
-        y = ops.attention_generic(x, x.shape[1], pg.k, pg.v, i32(pos), i32(seq_of), table, ps, window, scale, nh, nkv, d,
-                                  len(pos), vd=vd, chunk=chunk, softcap=cap, keep_first=keep_first, sinks=sk)
+        if tiled and all(n == 1 for n in sizes):
+            # steps of single tokens: the kernel for single queries, its keys split over two blocks where it may
+            y = ops.attention_decode(x, x.shape[1], pg.k, pg.v, i32(pos), table, ps, window, scale, nh, nkv, d, len(pos),
+                                     2 if max(pos) >= 128 else 1, chunk=chunk, softcap=cap, keep_first=keep_first, sinks=sk)
+        elif tiled:
+            y = ops.attention_prefill(x, x.shape[1], pg.k, pg.v, i32(pos), tiles_of(sizes, tiled), table, ps, window, scale,
+                                      nh, nkv, d, len(pos), tile_rows=tiled, chunk=chunk, softcap=cap, keep_first=keep_first,
+                                      sinks=sk)
+        else:
+            y = ops.attention_generic(x, x.shape[1], pg.k, pg.v, i32(pos), i32(seq_of), table, ps, window, scale, nh, nkv, d,
+                                      len(pos), vd=vd, chunk=chunk, softcap=cap, keep_first=keep_first, sinks=sk)
         at = 0
         for s, n in zip(live, sizes):
             got[s].append(y[at:at + n].double().cpu())
@@ -176,6 +197,25 @@ def test_attention_with_caps_windows_kept_positions_runs_and_sinks(ops, dtype, r
             assert float((got[s] - want[s]).abs().max()) <= tol(dtype, want[s], 2e-5, 2e-2), (s, nh, rule)
 
 
+@pytest.mark.parametrize("rule", [r for r in RULES if not r.get("chunk")] + [dict(window=100, keep_first=70, cap=4.0, sink=True),
+                                                                               dict(window=64, keep_first=64), dict(chunk=64, cap=3.0)])
+@pytest.mark.parametrize("rows", [16, 32])
+def test_tiled_prompt_attention_with_caps_windows_kept_positions_and_sinks(ops, rule, rows):
+    """The prompt kernel on the matrix cores: sequences long enough for several steps of 64 keys, fed whole, in long
+    portions and in short ones beside single tokens."""
+    rule = dict(rule)
+    for nh, nkv, d, ps in ((4, 2, 64, 16), (2, 2, 32, 8), (8, 2, 128, 16), (6, 1, 64, 4)):
+        if rows == 32 and nh // nkv > 4:
+            continue
+        sinks = torch.linspace(-2.0, 3.0, nh) if rule.get("sink") else None
+        kw = {k: v for k, v in rule.items() if k != "sink"}
+        lens = [230, 1, 97, 40]
+        cuts = [[100, 64, 1, 33, 30, 1, 1], [1], [97], [2, 17, 1, 1, 17, 1, 1]]
+        got, want = attention_case(ops, torch.bfloat16, nh, nkv, d, d, lens, cuts, ps=ps, sinks=sinks, seed=nh + d, tiled=rows, **kw)
+        for s in range(len(lens)):
+            assert float((got[s] - want[s]).abs().max()) <= tol(torch.bfloat16, want[s], 2e-5, 2e-2), (s, nh, d, rule)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("ps", [8, 16])
 def test_a_key_that_stands_out_is_seen_or_not_at_every_edge(ops, dtype, ps):
@@ -200,6 +240,14 @@ def test_a_key_that_stands_out_is_seen_or_not_at_every_edge(ops, dtype, ps):
             quiet, _ = attention_case(ops, dtype, nh, nkv, d, vd, [T], [[T]], ps=ps, scale=1.0, seed=3, **rule)
             moved = float((got[0][query, :vd] - quiet[0][query, :vd]).abs().max())
             assert (moved > 0.05) == seen, (kind, place, moved)
+            if dtype == torch.bfloat16:
+                # the same through the prompt kernel on the matrix cores (heads of 32), whole and in two portions
+                for cuts in ([[T]], [[query - 70, 71]], [[query, 1]], [[query - 80] + [1] * 81]):
+                    tg, tw = attention_case(ops, dtype, nh, nkv, 32, 32, [T], cuts, ps=ps, scale=1.0, seed=3, tiled=16,
+                                            plant=(0, place, query, 12.0), **rule)
+                    assert float((tg[0] - tw[0]).abs().max()) <= tol(dtype, tw[0], 2e-5, 2e-2), ("tiled", kind, place)
+                tq, _ = attention_case(ops, dtype, nh, nkv, 32, 32, [T], [[T]], ps=ps, scale=1.0, seed=3, tiled=16, **rule)
+                assert (float((tg[0][query, :32] - tq[0][query, :32]).abs().max()) > 0.05) == seen, ("tiled", kind, place)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
