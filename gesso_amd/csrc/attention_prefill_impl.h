@@ -256,8 +256,16 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
     else step_as(stage, std::false_type{}, k0);
   };
 
-  // One walk over the keys range_first .. range_last: by windows of pages, the sets of wavefronts taking the steps in turn.
-  auto walk = [&](int range_first, int range_last) {
+  // Two walks over keys, the same code for both (one copy of the steps: their row registers stay registers).  First the
+  // kept first positions that lie before the first key of the tile's window, where there are any: no query's window
+  // counts there (every one of these keys is before every query's window, and all of them are kept).  Then the
+  // window's keys first_key .. last_key.  Each walk goes by windows of pages, the sets of wavefronts taking the steps in
+  // turn.
+  const int kept_end = (keep_first > 0 && window > 0) ? (keep_first < first_key ? keep_first : first_key) : 0;
+  for (int pass = kept_end > 0 ? 0 : 1; pass < 2; ++pass) {
+    const int range_first = pass ? first_key : 0, range_last = pass ? last_key : kept_end - 1;
+#pragma unroll
+    for (int t = 0; t < QT; ++t) lo[t] = pass ? lo_own[t] : -(1 << 30);
     const int b0 = (int)__umulhi((unsigned)range_first, page_magic), b1 = (int)__umulhi((unsigned)range_last, page_magic);
     for (win_blk = b0; win_blk <= b1; win_blk += PF_MAXPAGES) {
       const int wend = win_blk + PF_MAXPAGES - 1 < b1 ? win_blk + PF_MAXPAGES - 1 : b1;
@@ -280,18 +288,7 @@ __global__ __launch_bounds__(G * KSPLIT * 64) void attention_prefill_kernel(
         step(std::integral_constant<int, 2>{}, k0 + 2 * STRIDE);
       }
     }
-  };
-  // the kept first positions that lie before the first key of the tile's window: a walk of their own, in which no
-  // query's window counts (every one of these keys is before every query's window, and all of them are kept)
-  const int kept_end = (keep_first > 0 && window > 0) ? (keep_first < first_key ? keep_first : first_key) : 0;
-  if (kept_end > 0) {
-#pragma unroll
-    for (int t = 0; t < QT; ++t) lo[t] = -(1 << 30);
-    walk(0, kept_end - 1);
-#pragma unroll
-    for (int t = 0; t < QT; ++t) lo[t] = lo_own[t];
   }
-  walk(first_key, last_key);
   if (KSPLIT > 1) {
     // add up the sets, in set order: set 0 takes the others' (reference point, sum, accumulator) through LDS,
     // one tile of queries at a time

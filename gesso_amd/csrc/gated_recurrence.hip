@@ -12,11 +12,12 @@
 // The decays are float32 rows (T, lda): a_t of head h at [oa + h] or, per channel, at [oa + h n, ...); beta_t float32 at
 // [ob + h] of rows (T, ldb).  Nothing is rounded below float32 between the rows and the output (T, H m).
 //
-// gated_state_scan: one block per (sequence, head, tile of 64 value columns).  Thread (rg, jl) = (tid & 3, tid >> 2)
-// holds the state's rows rg, rg + 4, ... of column jl in registers; the four partial sums of a column (S^T k, S^T q)
-// are neighbours in a wavefront.  A step's tokens come through LDS eight at a time.  Every sum runs in one fixed
-// order, whatever the step's cut: a sequence fed whole, in portions or token by token leaves the same state and
-// outputs, bit for bit.  A step of single tokens is the same kernel with one token a block.
+// gated_state_scan: one block per (sequence, head, tile of 32 value columns).  Thread (rg, jl) = (tid & 7, tid >> 3)
+// holds the state's rows rg, rg + 8, ... of column jl in registers; the eight partial sums of a column (S^T k, S^T q)
+// are neighbours in a wavefront and are added by moves between lanes.  A step's tokens come through LDS sixteen (wide
+// keys: eight) at a time, the next batch asked for while this one is computed.  Every sum runs in one fixed order,
+// whatever the step's cut: a sequence fed whole, in portions or token by token leaves the same state and outputs, bit
+// for bit.  A step of single tokens is the same kernel with one token a block.
 //
 // delta_rule_prep: what the gated delta rule computes between its convolutions and the recurrence, in float32:
 //   q <- q / sqrt(sum q^2 + unit_eps) * q_scale,  k <- k / sqrt(sum k^2 + unit_eps)        per (token, q/k head), in place
@@ -24,25 +25,40 @@
 // channel_decay: alpha = sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau), elementwise in place.
 #include "common.h"
 
-#define GR_TB 8          // tokens staged at once
-#define GR_COLS 64       // value columns a block
+#define GR_RG 8           // lanes that share a state column (each holds every eighth row of it)
+#define GR_COLS 32        // value columns a block (256 threads / GR_RG)
 
 __device__ __forceinline__ float gr_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
+// The sum over the eight neighbouring lanes that share a column: moves within quads, then the mirror of eight lanes
+// (lane i <-> 7 - i, which lies in the other quad); no trip through LDS.  Every lane gets the sum; its order is fixed.
+__device__ __forceinline__ float gr_sum8(float x) {
+  x += dpp_move<0xB1>(x);    // quad_perm [1,0,3,2]
+  x += dpp_move<0x4E>(x);    // quad_perm [2,3,0,1]
+  x += dpp_move<0x141>(x);   // row_half_mirror
+  return x;
+}
+
+// RMAX: state rows a thread (keys up to 8 RMAX wide).  A thread's rows i = rg + 8 r lie side by side in LDS (place
+// rg RMAX + r), so that it reads them sixteen bytes at a time.  The tokens of the next batch are asked for before this
+// batch is computed and land in registers meanwhile.
 template <typename TI, int RMAX, bool VEC, bool DELTA>
 __global__ void __launch_bounds__(256)
 gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov, int rep, float q_scale,
                         const float* __restrict__ decay, int lda, int oa, const float* __restrict__ beta, int ldb,
                         int ob, float* __restrict__ state, const int* __restrict__ q_start,
                         const int* __restrict__ slots, float* __restrict__ out, int H, int n, int m) {
-  constexpr int NMAX = 4 * RMAX;
-  __shared__ float qs[GR_TB][NMAX];
-  __shared__ float ks[GR_TB][NMAX];
-  __shared__ float al[VEC ? GR_TB : 1][VEC ? NMAX : 1];
-  __shared__ float vs[GR_TB][GR_COLS];
-  __shared__ float a1[GR_TB], bs[GR_TB];
+  constexpr int NMAX = GR_RG * RMAX;
+  constexpr int TB = NMAX <= 128 ? 16 : 8;                 // tokens staged at once
+  constexpr int PER = (TB * NMAX + 255) / 256;             // values of q (k, decays) a thread stages
+  constexpr int PERV = (TB * GR_COLS + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float qs[TB][NMAX];
+  __shared__ __attribute__((aligned(16))) float ks[TB][NMAX];
+  __shared__ __attribute__((aligned(16))) float al[VEC ? TB : 1][VEC ? NMAX : 4];
+  __shared__ float vs[TB][GR_COLS];
+  __shared__ float a1[TB], bs[TB];
   const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * GR_COLS;
-  const int tid = threadIdx.x, rg = tid & 3, jl = tid >> 2, j = j0 + jl;
+  const int tid = threadIdx.x, rg = tid & (GR_RG - 1), jl = tid / GR_RG, j = j0 + jl;
   const int t0 = q_start[seq], t1 = q_start[seq + 1];
   if (t1 <= t0) return;
   const int hq = h / rep;
@@ -50,62 +66,99 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
   float s[RMAX];
 #pragma unroll
   for (int r = 0; r < RMAX; ++r) {
-    const int i = rg + 4 * r;
+    const int i = rg + GR_RG * r;
     s[r] = (i < n && j < m) ? S[(size_t)i * m + j] : 0.f;
   }
-  for (int tb = t0; tb < t1; tb += GR_TB) {
-    const int nb = t1 - tb < GR_TB ? t1 - tb : GR_TB;
-    __syncthreads();                                   // the batch before has been read
-    for (int idx = tid; idx < nb * n; idx += 256) {
+  // a batch's values on their way: asked for one batch ahead, kept in registers until the batch before has been read
+  float rq[PER], rk[PER], ra[VEC ? PER : 1], rv[PERV], r1 = 0.f, rb = 0.f;
+  auto ask = [&](int tb) {
+    const int nb = t1 - tb < TB ? t1 - tb : TB;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int idx = tid + u * 256;
       const int tt = idx / n, i = idx - tt * n;
-      const TI* row = x + (size_t)(tb + tt) * ld;
-      qs[tt][i] = to_f32(row[oq + hq * n + i]) * q_scale;
-      ks[tt][i] = to_f32(row[ok + hq * n + i]);
-      if (VEC) al[tt][i] = decay[(size_t)(tb + tt) * lda + oa + h * n + i];
+      const bool live = idx < nb * n;
+      const TI* row = x + (size_t)(tb + (live ? tt : 0)) * ld;
+      rq[u] = live ? to_f32(row[oq + hq * n + i]) * q_scale : 0.f;
+      rk[u] = live ? to_f32(row[ok + hq * n + i]) : 0.f;
+      if (VEC) ra[u] = live ? decay[(size_t)(tb + tt) * lda + oa + h * n + i] : 0.f;
     }
-    for (int idx = tid; idx < nb * GR_COLS; idx += 256) {
+#pragma unroll
+    for (int u = 0; u < PERV; ++u) {
+      const int idx = tid + u * 256;
       const int tt = idx / GR_COLS, c = idx - tt * GR_COLS;
-      vs[tt][c] = j0 + c < m ? to_f32(x[(size_t)(tb + tt) * ld + ov + h * m + j0 + c]) : 0.f;
+      rv[u] = (idx < nb * GR_COLS && j0 + c < m) ? to_f32(x[(size_t)(tb + tt) * ld + ov + h * m + j0 + c]) : 0.f;
     }
     if (tid < nb) {
-      if (!VEC) a1[tid] = decay[(size_t)(tb + tid) * lda + oa + h];
-      if (DELTA) bs[tid] = beta[(size_t)(tb + tid) * ldb + ob + h];
+      if (!VEC) r1 = decay[(size_t)(tb + tid) * lda + oa + h];
+      if (DELTA) rb = beta[(size_t)(tb + tid) * ldb + ob + h];
     }
+  };
+  auto put = [&](int tb) {
+    const int nb = t1 - tb < TB ? t1 - tb : TB;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < nb * n) {
+        const int tt = idx / n, i = idx - tt * n;
+        const int place = (i & (GR_RG - 1)) * RMAX + (i >> 3);
+        qs[tt][place] = rq[u];
+        ks[tt][place] = rk[u];
+        if (VEC) al[tt][place] = ra[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < PERV; ++u) {
+      const int idx = tid + u * 256;
+      if (idx < nb * GR_COLS) vs[idx / GR_COLS][idx % GR_COLS] = rv[u];
+    }
+    if (tid < nb) {
+      if (!VEC) a1[tid] = r1;
+      if (DELTA) bs[tid] = rb;
+    }
+  };
+  // rows this thread holds that lie beyond n (the last ones, where n is no multiple of 8) stay zero: their places in
+  // LDS are never written, so what is read there is multiplied into nothing only if it is finite; they are masked
+  const int live_rows = (n - rg + GR_RG - 1) / GR_RG;      // rows r < live_rows exist
+  ask(t0);
+  for (int tb = t0; tb < t1; tb += TB) {
+    const int nb = t1 - tb < TB ? t1 - tb : TB;
+    __syncthreads();                                   // the batch before has been read
+    put(tb);
     __syncthreads();
+    if (tb + TB < t1) ask(tb + TB);
     for (int tt = 0; tt < nb; ++tt) {
       float u = vs[tt][jl];
       const float a = VEC ? 0.f : a1[tt];
-      float answered = 0.f;
+      const float* kr = &ks[tt][rg * RMAX];
+      const float* qr = &qs[tt][rg * RMAX];
+      const float* ar = &al[VEC ? tt : 0][VEC ? rg * RMAX : 0];
+      float kv[RMAX];
+      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
       for (int r = 0; r < RMAX; ++r) {
-        const int i = rg + 4 * r;
-        if (i < n) {
-          s[r] *= VEC ? al[tt][i] : a;
-          if (DELTA) answered = fmaf(s[r], ks[tt][i], answered);
+        kv[r] = r < live_rows ? kr[r] : 0.f;
+        s[r] *= VEC ? (r < live_rows ? ar[r] : 0.f) : a;
+        if (DELTA) {
+          const float t = s[r] * kv[r];
+          if ((r & 3) == 0) p0 += t; else if ((r & 3) == 1) p1 += t; else if ((r & 3) == 2) p2 += t; else p3 += t;
         }
       }
-      if (DELTA) {
-        answered += __shfl_xor(answered, 1, 64);
-        answered += __shfl_xor(answered, 2, 64);
-        u = bs[tt] * (u - answered);
-      }
-      float part = 0.f;
+      if (DELTA) u = bs[tt] * (u - gr_sum8((p0 + p1) + (p2 + p3)));
+      p0 = p1 = p2 = p3 = 0.f;
 #pragma unroll
       for (int r = 0; r < RMAX; ++r) {
-        const int i = rg + 4 * r;
-        if (i < n) {
-          s[r] = fmaf(ks[tt][i], u, s[r]);
-          part = fmaf(s[r], qs[tt][i], part);
-        }
+        s[r] = fmaf(kv[r], u, s[r]);
+        const float t = s[r] * (r < live_rows ? qr[r] : 0.f);
+        if ((r & 3) == 0) p0 += t; else if ((r & 3) == 1) p1 += t; else if ((r & 3) == 2) p2 += t; else p3 += t;
       }
-      part += __shfl_xor(part, 1, 64);
-      part += __shfl_xor(part, 2, 64);
+      const float part = gr_sum8((p0 + p1) + (p2 + p3));
       if (rg == 0 && j < m) out[((size_t)(tb + tt) * H + h) * m + j] = part;
     }
   }
 #pragma unroll
   for (int r = 0; r < RMAX; ++r) {
-    const int i = rg + 4 * r;
+    const int i = rg + GR_RG * r;
     if (i < n && j < m) S[(size_t)i * m + j] = s[r];
   }
 }
@@ -130,10 +183,10 @@ extern "C" int gs_gated_state_scan(const void* x, int dtype, int ld, int oq, int
   gated_state_scan_kernel<TI, R, V, D><<<grid, 256, 0, stream>>>((const TI*)x, ld, oq, ok, ov, rep, q_scale, decay, \
                                                                  lda, oa, beta, ldb, ob, state, q_start, slots, out, H, n, m)
 #define GR_RUN_R(TI, V, D)                   \
-  if (n <= 32) GR_RUN(TI, 8, V, D);          \
-  else if (n <= 64) GR_RUN(TI, 16, V, D);    \
-  else if (n <= 128) GR_RUN(TI, 32, V, D);   \
-  else GR_RUN(TI, 64, V, D)
+  if (n <= 32) GR_RUN(TI, 4, V, D);          \
+  else if (n <= 64) GR_RUN(TI, 8, V, D);     \
+  else if (n <= 128) GR_RUN(TI, 16, V, D);   \
+  else GR_RUN(TI, 32, V, D)
 #define GR_RUN_T(TI)                                      \
   if (per_channel && beta) { GR_RUN_R(TI, true, true); }  \
   else if (per_channel) { GR_RUN_R(TI, true, false); }    \
