@@ -12,8 +12,8 @@
 // The decays are float32 rows (T, lda): a_t of head h at [oa + h] or, per channel, at [oa + h n, ...); beta_t float32 at
 // [ob + h] of rows (T, ldb).  Nothing is rounded below float32 between the rows and the output (T, H m).
 //
-// gated_state_scan: one block per (sequence, head, tile of 32 value columns).  Thread (rg, jl) = (tid & 7, tid >> 3)
-// holds the state's rows rg, rg + 8, ... of column jl in registers; the eight partial sums of a column (S^T k, S^T q)
+// gated_state_scan: one block per (sequence, head, tile of 16 value columns).  Thread (rg, jl) = (tid & 15, tid >> 4)
+// holds the state's rows rg, rg + 16, ... of column jl in registers; the sixteen partial sums of a column (S^T k, S^T q)
 // are neighbours in a wavefront and are added by moves between lanes.  A step's tokens come through LDS sixteen (wide
 // keys: eight) at a time, the next batch asked for while this one is computed.  Every sum runs in one fixed order,
 // whatever the step's cut: a sequence fed whole, in portions or token by token leaves the same state and outputs, bit
@@ -25,22 +25,24 @@
 // channel_decay: alpha = sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau), elementwise in place.
 #include "common.h"
 
-#define GR_RG 8           // lanes that share a state column (each holds every eighth row of it)
-#define GR_COLS 32        // value columns a block (256 threads / GR_RG)
+#define GR_RG 16          // lanes that share a state column (each holds every sixteenth row of it)
+#define GR_COLS 16        // value columns a block (256 threads / GR_RG)
 
 __device__ __forceinline__ float gr_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-// The sum over the eight neighbouring lanes that share a column: moves within quads, then the mirror of eight lanes
-// (lane i <-> 7 - i, which lies in the other quad); no trip through LDS.  Every lane gets the sum; its order is fixed.
-__device__ __forceinline__ float gr_sum8(float x) {
+// The sum over the sixteen neighbouring lanes that share a column (a row of lanes): moves within quads, then the
+// mirrors of eight and of sixteen lanes (lane i <-> 7 - i, then i <-> 15 - i, which lie in parts not yet added); no trip
+// through LDS.  Every lane gets the sum; its order is fixed.
+__device__ __forceinline__ float gr_sum16(float x) {
   x += dpp_move<0xB1>(x);    // quad_perm [1,0,3,2]
   x += dpp_move<0x4E>(x);    // quad_perm [2,3,0,1]
   x += dpp_move<0x141>(x);   // row_half_mirror
+  x += dpp_move<0x140>(x);   // row_mirror
   return x;
 }
 
-// RMAX: state rows a thread (keys up to 8 RMAX wide).  A thread's rows i = rg + 8 r lie side by side in LDS (place
-// rg RMAX + r), so that it reads them sixteen bytes at a time.  The tokens of the next batch are asked for before this
+// RMAX: state rows a thread (keys up to 16 RMAX wide).  A thread's rows i = rg + 16 r lie side by side in LDS (place
+// rg RMAX + r), so that it reads them up to sixteen bytes at a time; the places of rows beyond n hold zeros.  The tokens of the next batch are asked for before this
 // batch is computed and land in registers meanwhile.
 template <typename TI, int RMAX, bool VEC, bool DELTA>
 __global__ void __launch_bounds__(256)
@@ -101,7 +103,7 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
       const int idx = tid + u * 256;
       if (idx < nb * n) {
         const int tt = idx / n, i = idx - tt * n;
-        const int place = (i & (GR_RG - 1)) * RMAX + (i >> 3);
+        const int place = (i & (GR_RG - 1)) * RMAX + (i >> 4);
         qs[tt][place] = rq[u];
         ks[tt][place] = rk[u];
         if (VEC) al[tt][place] = ra[u];
@@ -117,9 +119,52 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
       if (DELTA) bs[tid] = rb;
     }
   };
-  // rows this thread holds that lie beyond n (the last ones, where n is no multiple of 8) stay zero: their places in
-  // LDS are never written, so what is read there is multiplied into nothing only if it is finite; they are masked
-  const int live_rows = (n - rg + GR_RG - 1) / GR_RG;      // rows r < live_rows exist
+  // the places of rows beyond n (where n is no multiple of 16) are written here once and never again: such a row of
+  // the state starts at zero and stays there, whatever stands beside it
+  for (int idx = tid; idx < TB * NMAX; idx += 256) {
+    qs[idx / NMAX][idx % NMAX] = 0.f;
+    ks[idx / NMAX][idx % NMAX] = 0.f;
+    if (VEC) al[idx / NMAX][idx % NMAX] = 0.f;
+  }
+  struct Tok {
+    float k[RMAX], q[RMAX], a[VEC ? RMAX : 1];
+    float v, a1, b;
+  };
+  auto take = [&](Tok& t, int tt) __attribute__((always_inline)) {
+    const float* kr = &ks[tt][rg * RMAX];
+    const float* qr = &qs[tt][rg * RMAX];
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      t.k[r] = kr[r];
+      t.q[r] = qr[r];
+      if (VEC) t.a[r] = al[tt][rg * RMAX + r];
+    }
+    t.v = vs[tt][jl];
+    t.a1 = VEC ? 0.f : a1[tt];
+    t.b = DELTA ? bs[tt] : 0.f;
+  };
+  auto advance = [&](const Tok& t, int row) __attribute__((always_inline)) {
+    float u = t.v;
+    float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      s[r] *= VEC ? t.a[r] : t.a1;
+      if (DELTA) {
+        const float w = s[r] * t.k[r];
+        if ((r & 3) == 0) p0 += w; else if ((r & 3) == 1) p1 += w; else if ((r & 3) == 2) p2 += w; else p3 += w;
+      }
+    }
+    if (DELTA) u = t.b * (u - gr_sum16((p0 + p1) + (p2 + p3)));
+    p0 = p1 = p2 = p3 = 0.f;
+#pragma unroll
+    for (int r = 0; r < RMAX; ++r) {
+      s[r] = fmaf(t.k[r], u, s[r]);
+      const float w = s[r] * t.q[r];
+      if ((r & 3) == 0) p0 += w; else if ((r & 3) == 1) p1 += w; else if ((r & 3) == 2) p2 += w; else p3 += w;
+    }
+    const float part = gr_sum16((p0 + p1) + (p2 + p3));
+    if (rg == 0 && j < m) out[((size_t)row * H + h) * m + j] = part;
+  };
   ask(t0);
   for (int tb = t0; tb < t1; tb += TB) {
     const int nb = t1 - tb < TB ? t1 - tb : TB;
@@ -127,33 +172,17 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
     put(tb);
     __syncthreads();
     if (tb + TB < t1) ask(tb + TB);
-    for (int tt = 0; tt < nb; ++tt) {
-      float u = vs[tt][jl];
-      const float a = VEC ? 0.f : a1[tt];
-      const float* kr = &ks[tt][rg * RMAX];
-      const float* qr = &qs[tt][rg * RMAX];
-      const float* ar = &al[VEC ? tt : 0][VEC ? rg * RMAX : 0];
-      float kv[RMAX];
-      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
-#pragma unroll
-      for (int r = 0; r < RMAX; ++r) {
-        kv[r] = r < live_rows ? kr[r] : 0.f;
-        s[r] *= VEC ? (r < live_rows ? ar[r] : 0.f) : a;
-        if (DELTA) {
-          const float t = s[r] * kv[r];
-          if ((r & 3) == 0) p0 += t; else if ((r & 3) == 1) p1 += t; else if ((r & 3) == 2) p2 += t; else p3 += t;
-        }
+    // A token's operands come from LDS one token ahead (two sets of registers, used in turn), so that their way from
+    // LDS lies behind the token before; the chain from state to state is all that a token waits for.
+    Tok ta, tb2;
+    take(ta, 0);
+    for (int tt = 0; tt < nb; tt += 2) {
+      if (tt + 1 < nb) take(tb2, tt + 1);
+      advance(ta, tb + tt);
+      if (tt + 1 < nb) {
+        if (tt + 2 < nb) take(ta, tt + 2);
+        advance(tb2, tb + tt + 1);
       }
-      if (DELTA) u = bs[tt] * (u - gr_sum8((p0 + p1) + (p2 + p3)));
-      p0 = p1 = p2 = p3 = 0.f;
-#pragma unroll
-      for (int r = 0; r < RMAX; ++r) {
-        s[r] = fmaf(kv[r], u, s[r]);
-        const float t = s[r] * (r < live_rows ? qr[r] : 0.f);
-        if ((r & 3) == 0) p0 += t; else if ((r & 3) == 1) p1 += t; else if ((r & 3) == 2) p2 += t; else p3 += t;
-      }
-      const float part = gr_sum8((p0 + p1) + (p2 + p3));
-      if (rg == 0 && j < m) out[((size_t)(tb + tt) * H + h) * m + j] = part;
     }
   }
 #pragma unroll
@@ -183,10 +212,10 @@ extern "C" int gs_gated_state_scan(const void* x, int dtype, int ld, int oq, int
   gated_state_scan_kernel<TI, R, V, D><<<grid, 256, 0, stream>>>((const TI*)x, ld, oq, ok, ov, rep, q_scale, decay, \
                                                                  lda, oa, beta, ldb, ob, state, q_start, slots, out, H, n, m)
 #define GR_RUN_R(TI, V, D)                   \
-  if (n <= 32) GR_RUN(TI, 4, V, D);          \
-  else if (n <= 64) GR_RUN(TI, 8, V, D);     \
-  else if (n <= 128) GR_RUN(TI, 16, V, D);   \
-  else GR_RUN(TI, 32, V, D)
+  if (n <= 32) GR_RUN(TI, 2, V, D);          \
+  else if (n <= 64) GR_RUN(TI, 4, V, D);     \
+  else if (n <= 128) GR_RUN(TI, 8, V, D);    \
+  else GR_RUN(TI, 16, V, D)
 #define GR_RUN_T(TI)                                      \
   if (per_channel && beta) { GR_RUN_R(TI, true, true); }  \
   else if (per_channel) { GR_RUN_R(TI, true, false); }    \
