@@ -6,6 +6,14 @@ into the request's pages and the queries read all keys they may see from there.
 Reference: ``src/Inference/Inference.jl:296-357`` (order of norm and rotation ``:307-323``),
 causal rule ``:1206-1207``, grouping ``:1852-1870``.  The cache holds post-norm, post-rotation
 keys and raw values (``:2417-2422``).  Wq, Wk, Wv are laid side by side at load.
+
+What a spec may ask for beyond that, each off unless said: values of their own width, runs of positions, a sink term
+``exp(0)`` and values cached turned; a head norm without a weight; biases on the input products alone; scores capped by
+``cap tanh(score / cap)``; with a window, first positions of the sequence that stay visible beyond it; a sink of each
+head's own, ``exp(s_h)`` with ``s_h`` stored; a gate on the heads, ``sigmoid(W_g x)`` (or silu), whose product rides
+behind q, k and v in the one weight; values shared between the mixers that say so (the first to run in a step keeps
+its own, each later one caches ``(1 - m) v + m v_first``).  A mixer with any of these is not ``plain``: it goes through
+the kernels that know the rules it uses (the general kernel knows them all).
 """
 from __future__ import annotations
 
