@@ -126,7 +126,9 @@ def kuditar_spec(cfg: KuditarConfig) -> ModelSpec:
     return ModelSpec(architecture=ARCHITECTURE, hidden=W, vocab=cfg.vocab, blocks=tuple(blocks),
                      schedule=tuple(LayerCall(i) for i in range(len(blocks))), final_norm=norm, tie_embeddings=True,
                      max_position=cfg.max_position, names=names, embed_scale=cfg.embedding_scale,
-                     ignored_tensors=(".norm2", ".norm2.b"))
+                     # (a file may hold the second norm of a layer without a feed-forward, or the share of a layer
+                     # that blends nothing: nobody reads them)
+                     ignored_tensors=(".norm2", ".norm2.b", ".vmix"))
 
 
 register_architecture(ARCHITECTURE, KuditarConfig.from_dict, kuditar_spec, KuditarConfig.to_json, complete=complete)
