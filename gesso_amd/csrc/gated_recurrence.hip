@@ -19,6 +19,13 @@
 // whatever the step's cut: a sequence fed whole, in portions or token by token leaves the same state and outputs, bit
 // for bit.  A step of single tokens is the same kernel with one token a block.
 //
+// Long portions, segment by segment.  Over a run of tokens the state goes S -> M S + B with an n x n matrix M (what the
+// decays and the delta rule's corrections do to a state, whatever it holds) and B (what the run writes, starting from
+// nothing).  So the segments of a long portion run side by side: the same kernel gives every segment's B (from a state
+// of zeros) and M (from the identity, with every value zero), gated_state_chain walks a sequence's segments in order
+// (S_(s+1) = M_s S_s + B_s, a product of n x n by n x 16 a block and segment) and leaves every segment's first state,
+// and the kernel runs once more from those states for the outputs.  The same arithmetic in another association.
+//
 // delta_rule_prep: what the gated delta rule computes between its convolutions and the recurrence, in float32:
 //   q <- q / sqrt(sum q^2 + unit_eps) * q_scale,  k <- k / sqrt(sum k^2 + unit_eps)        per (token, q/k head), in place
 //   g = exp(-exp(A_log[h]) softplus(a + dt_bias[h])),  beta = sigmoid(b)                     per (token, head)
@@ -89,7 +96,7 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
     for (int u = 0; u < PERV; ++u) {
       const int idx = tid + u * 256;
       const int tt = idx / GR_COLS, c = idx - tt * GR_COLS;
-      rv[u] = (idx < nb * GR_COLS && j0 + c < m) ? to_f32(x[(size_t)(tb + tt) * ld + ov + h * m + j0 + c]) : 0.f;
+      rv[u] = (ov >= 0 && idx < nb * GR_COLS && j0 + c < m) ? to_f32(x[(size_t)(tb + tt) * ld + ov + h * m + j0 + c]) : 0.f;
     }
     if (tid < nb) {
       if (!VEC) r1 = decay[(size_t)(tb + tid) * lda + oa + h];
@@ -163,7 +170,7 @@ gated_state_scan_kernel(const TI* __restrict__ x, int ld, int oq, int ok, int ov
       if ((r & 3) == 0) p0 += w; else if ((r & 3) == 1) p1 += w; else if ((r & 3) == 2) p2 += w; else p3 += w;
     }
     const float part = gr_sum16((p0 + p1) + (p2 + p3));
-    if (rg == 0 && j < m) out[((size_t)row * H + h) * m + j] = part;
+    if (out && rg == 0 && j < m) out[((size_t)row * H + h) * m + j] = part;
   };
   ask(t0);
   for (int tb = t0; tb < t1; tb += TB) {
@@ -201,7 +208,8 @@ extern "C" int gs_gated_state_scan(const void* x, int dtype, int ld, int oq, int
   GS_REQUIRE(qk_heads > 0 && H % qk_heads == 0, "gated_state_scan: %d heads do not share %d queries and keys evenly", H,
              qk_heads);
   GS_REQUIRE(H <= 65535 && (m + GR_COLS - 1) / GR_COLS <= 65535, "gated_state_scan: too many heads or value columns");
-  GS_REQUIRE(oq >= 0 && ok >= 0 && ov >= 0 && oq + qk_heads * n <= ld && ok + qk_heads * n <= ld && ov + H * m <= ld,
+  // (ov < 0: every value is zero, what the state does to itself over the tokens; out null: the states alone are wanted)
+  GS_REQUIRE(oq >= 0 && ok >= 0 && oq + qk_heads * n <= ld && ok + qk_heads * n <= ld && (ov < 0 || ov + H * m <= ld),
              "gated_state_scan: q, k or v lie outside the rows of %d", ld);
   GS_REQUIRE(decay && oa >= 0 && oa + (per_channel ? H * n : H) <= lda, "gated_state_scan: the decays lie outside their rows of %d", lda);
   GS_REQUIRE(!beta || (ob >= 0 && ob + H <= ldb), "gated_state_scan: the write strengths lie outside their rows of %d", ldb);
@@ -232,6 +240,117 @@ extern "C" int gs_gated_state_scan(const void* x, int dtype, int ld, int oq, int
 #undef GR_RUN_R
 #undef GR_RUN
   GS_LAUNCH_CHECK("gated_state_scan");
+  return 0;
+}
+
+// One block per (sequence, head, 16 value columns): S (n x 16) in LDS; for the sequence's segments in order, the state a
+// segment starts from goes to `first`, then S <- M_seg S + B_seg; the last state is the request's.  M (segments, H, n, n),
+// B and first (segments, H, n, m), state (slots, H, n, m); seq_seg (nseq + 1): where each sequence's segments begin.
+// M comes through LDS in tiles of R rows (R n <= 4096 values, R a multiple of 16 or n itself), read with 16-byte loads
+// one tile ahead of the products that use it (the walk is a chain of small steps: what it waits for is memory), and so
+// do the rows of B.
+#define GR_CHAIN_TILE 4096
+__global__ void __launch_bounds__(256)
+gated_state_chain_kernel(const float* __restrict__ M, const float* __restrict__ B, float* __restrict__ first,
+                         float* __restrict__ state, const int* __restrict__ seq_seg, const int* __restrict__ slots, int H,
+                         int n, int m, int R) {
+  extern __shared__ float ch_s[];             // S and its successor, n x 16 each; then a tile of M, R x n
+  float* S = ch_s;
+  float* N = ch_s + (size_t)n * GR_COLS;
+  float* Mt = ch_s + 2 * (size_t)n * GR_COLS;
+  const int seq = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * GR_COLS;
+  const int tid = threadIdx.x, jl = tid & (GR_COLS - 1), rl = tid / GR_COLS, j = j0 + jl;
+  const int s0 = seq_seg[seq], s1 = seq_seg[seq + 1];
+  if (s1 <= s0) return;
+  float* own = state + (((size_t)slots[seq] * H + h) * n) * m;
+  for (int i = rl; i < n; i += 16) S[i * GR_COLS + jl] = j < m ? own[(size_t)i * m + j] : 0.f;
+  const int tps = (n + R - 1) / R, total = (s1 - s0) * tps;      // tiles a segment, tiles in all
+  const bool vec = (n & 3) == 0;                                   // (rows of M start at multiples of 16 bytes)
+  float pm[16], pb[4];
+  auto ask = [&](int t) {
+    const int sg = s0 + t / tps, r0 = (t % tps) * R;
+    const int len = (r0 + R < n ? R : n - r0) * n;
+    const float* src = M + (((size_t)sg * H + h) * n + r0) * n;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int at = (tid + 256 * u) * 4;
+      if (vec && at + 3 < len) {
+        const float4 v = *reinterpret_cast<const float4*>(src + at);
+        pm[4 * u] = v.x; pm[4 * u + 1] = v.y; pm[4 * u + 2] = v.z; pm[4 * u + 3] = v.w;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) pm[4 * u + e] = at + e < len ? src[at + e] : 0.f;
+      }
+    }
+    const float* bsrc = B + ((size_t)sg * H + h) * n * m;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = r0 + rl + 16 * r;
+      pb[r] = (rl + 16 * r < R && i < n && j < m) ? bsrc[(size_t)i * m + j] : 0.f;
+    }
+  };
+  ask(0);
+  for (int t = 0; t < total; ++t) {
+    const int sg = s0 + t / tps, r0 = (t % tps) * R;
+    __syncthreads();                          // the tile before has been read (and, at a segment's start, S is whole)
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int at = (tid + 256 * u) * 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (at + e < R * n) Mt[at + e] = pm[4 * u + e];
+    }
+    float bv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) bv[r] = pb[r];
+    __syncthreads();
+    if (t + 1 < total) ask(t + 1);
+    if (r0 == 0) {
+      float* Fs = first + ((size_t)sg * H + h) * n * m;
+      for (int i = rl; i < n; i += 16)
+        if (j < m) Fs[(size_t)i * m + j] = S[i * GR_COLS + jl];
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int ir = rl + 16 * r, i = r0 + ir;
+      if (ir < R && i < n) {
+        const float* row = Mt + (size_t)ir * n;
+        float a0 = bv[r], a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        int k = 0;
+        for (; k + 3 < n; k += 4) {
+          a0 = fmaf(row[k], S[k * GR_COLS + jl], a0);
+          a1 = fmaf(row[k + 1], S[(k + 1) * GR_COLS + jl], a1);
+          a2 = fmaf(row[k + 2], S[(k + 2) * GR_COLS + jl], a2);
+          a3 = fmaf(row[k + 3], S[(k + 3) * GR_COLS + jl], a3);
+        }
+        for (; k < n; ++k) a0 = fmaf(row[k], S[k * GR_COLS + jl], a0);
+        N[i * GR_COLS + jl] = (a0 + a1) + (a2 + a3);
+      }
+    }
+    if (r0 + R >= n) {                         // the segment's last tile: its successor is whole
+      __syncthreads();
+      float* x = S;
+      S = N;
+      N = x;
+    }
+  }
+  __syncthreads();
+  for (int i = rl; i < n; i += 16)
+    if (j < m) own[(size_t)i * m + j] = S[i * GR_COLS + jl];
+}
+
+extern "C" int gs_gated_state_chain(const float* M, const float* B, float* first, float* state, const int* seq_seg,
+                                    const int* slots, int nseq, int H, int n, int m, hipStream_t stream) {
+  GS_REQUIRE(nseq >= 0 && H > 0 && n > 0 && n <= 256 && m > 0, "gated_state_chain: bad sizes nseq=%d H=%d n=%d m=%d", nseq, H, n, m);
+  GS_REQUIRE(H <= 65535 && (m + GR_COLS - 1) / GR_COLS <= 65535, "gated_state_chain: too many heads or value columns");
+  if (nseq == 0) return 0;
+  // rows of M a tile: all of them where n x n values fit, else as many whole sixteens as do (n <= 256: at least 16)
+  int R = n * n <= GR_CHAIN_TILE ? n : (GR_CHAIN_TILE / n) / 16 * 16;
+  if (R > 64) R = 64;                          // (a thread keeps four rows of B for a tile)
+  dim3 grid(nseq, H, (m + GR_COLS - 1) / GR_COLS);
+  const size_t lds = (2 * (size_t)n * GR_COLS + (size_t)R * n) * sizeof(float);
+  gated_state_chain_kernel<<<grid, 256, lds, stream>>>(M, B, first, state, seq_seg, slots, H, n, m, R);
+  GS_LAUNCH_CHECK("gated_state_chain");
   return 0;
 }
 

@@ -1601,14 +1601,15 @@ GATED_STATE_MAX_KEY = 256
 
 def gated_state_scan(x, oq: int, ok: int, ov: int, H: int, qk_heads: int, n: int, m: int, decay, oa: int,
                      per_channel: bool, state, q_start, slots, nseq: int, q_scale: float = 1.0, beta=None, ob: int = 0,
-                     out: torch.Tensor = None) -> torch.Tensor:
+                     out: torch.Tensor = None, want_out: bool = True) -> torch.Tensor:
     """Per sequence and head ``S <- diag(a_t) S; u = beta_t (v_t - S^T k_t)`` (``u = v_t`` without ``beta``);
     ``S <- S + k_t u^T; o_t = S^T (q_scale q_t)``.
 
     ``x (T, ld)`` float32 or bfloat16 holds q of head ``h`` at ``[oq + (h // (H / qk_heads)) n, ...)``, k likewise from
-    ``ok``, v at ``[ov + h m, ...)``.  ``decay`` float32 rows: ``a_t`` of head ``h`` at ``[oa + h]``, or with
-    ``per_channel`` one a key channel at ``[oa + h n, ...)``.  ``beta`` float32 rows with head ``h`` at ``[ob + h]``.
-    ``state (slots, H, n, m)`` float32 is read and advanced.  Returns ``(T, H m)`` float32."""
+    ``ok``, v at ``[ov + h m, ...)`` (``ov`` < 0: every value is zero).  ``decay`` float32 rows: ``a_t`` of head ``h`` at
+    ``[oa + h]``, or with ``per_channel`` one a key channel at ``[oa + h n, ...)``.  ``beta`` float32 rows with head ``h``
+    at ``[ob + h]``.  ``state (slots, H, n, m)`` float32 is read and advanced.  Returns ``(T, H m)`` float32, or None
+    without ``want_out`` (the states alone are wanted)."""
     _dev(x, decay, beta, state, q_start, slots, out)
     _need(x.dim() == 2 and decay.dim() == 2 and decay.dtype == torch.float32 and decay.shape[0] == x.shape[0],
           "gated_state_scan: rows (T, ld) and float32 decay rows (T, lda)")
@@ -1620,13 +1621,56 @@ def gated_state_scan(x, oq: int, ok: int, ov: int, H: int, qk_heads: int, n: int
           "gated_state_scan: state must be float32 (slots, H, n, m)")
     _i32(q_start, nseq + 1, "q_start")
     _i32(slots, nseq, "slots")
-    if out is None:
-        out = torch.empty((T, H * m), dtype=torch.float32, device=x.device)
-    _need(out.shape == (T, H * m) and out.dtype == torch.float32, "gated_state_scan: out must be float32 (T, H m)")
+    if want_out:
+        if out is None:
+            out = torch.empty((T, H * m), dtype=torch.float32, device=x.device)
+        _need(out.shape == (T, H * m) and out.dtype == torch.float32, "gated_state_scan: out must be float32 (T, H m)")
+    else:
+        out = None
     _check(lib().gs_gated_state_scan(_p(x), _dt(x), ld, oq, ok, ov, qk_heads, float(q_scale), _p(decay), decay.shape[1], oa,
                                      1 if per_channel else 0, _p(beta), beta.shape[1] if beta is not None else 0, ob,
                                      _p(state), _p(q_start), _p(slots), _p(out), nseq, H, n, m, _stream()))
     return out
+
+
+def state_segment_tables(q_lens, seg_len: int, device):
+    """A step's portions cut into segments of at most ``seg_len`` tokens: int32 on the device, ``(where each segment's
+    tokens begin among the step's rows (segments + 1), where each sequence's segments begin (sequences + 1), the
+    segments' numbers (segments))``, and the number of segments."""
+    starts, first, at = [0], [0], 0
+    for L in q_lens:
+        for a in range(0, L, seg_len):
+            starts.append(at + min(a + seg_len, L))
+        at += L
+        first.append(len(starts) - 1)
+    nseg = len(starts) - 1
+    t = torch.tensor(starts + first + list(range(nseg)), dtype=torch.int32).pin_memory().to(device, non_blocking=True)
+    return t[:nseg + 1], t[nseg + 1:nseg + 1 + len(first)], t[nseg + 1 + len(first):], nseg
+
+
+def gated_state_scan_segments(x, oq: int, ok: int, ov: int, H: int, qk_heads: int, n: int, m: int, decay, oa: int,
+                              per_channel: bool, state, q_lens, slots, seg_len: int, q_scale: float = 1.0, beta=None,
+                              ob: int = 0) -> torch.Tensor:
+    """:func:`gated_state_scan` with the portions (``q_lens``: tokens of each sequence, on the host) cut into segments of
+    ``seg_len`` tokens that run side by side.  Over a segment the state goes ``S -> M S + B``: the kernel gives every
+    segment's ``B`` (from a state of zeros) and ``M`` (from the identity, every value zero); ``gated_state_chain`` walks
+    each sequence's segments in order, leaves every segment's first state and the request's new state; the kernel then
+    runs from those states for the outputs.  The same arithmetic in another association (float32 rounding apart)."""
+    _dev(state, slots)
+    nseq = len(q_lens)
+    seg_start, seq_seg, ids, nseg = state_segment_tables(q_lens, seg_len, x.device)
+    dev, f32 = x.device, torch.float32
+    B = torch.zeros((nseg, H, n, m), dtype=f32, device=dev)
+    M = torch.eye(n, dtype=f32, device=dev).expand(nseg, H, n, n).contiguous()
+    first = torch.empty((nseg, H, n, m), dtype=f32, device=dev)
+    args = (H, qk_heads, n)
+    kw = dict(q_scale=q_scale, beta=beta, ob=ob)
+    gated_state_scan(x, oq, ok, ov, *args, m, decay, oa, per_channel, B, seg_start, ids, nseg, want_out=False, **kw)
+    gated_state_scan(x, oq, ok, -1, *args, n, decay, oa, per_channel, M, seg_start, ids, nseg, want_out=False, **kw)
+    _i32(slots, nseq, "slots")
+    _need(state.dtype == f32 and state.dim() == 4 and state.shape[1:] == (H, n, m), "gated_state_scan: state must be float32 (slots, H, n, m)")
+    _check(lib().gs_gated_state_chain(_p(M), _p(B), _p(first), _p(state), _p(seq_seg), _p(slots), nseq, H, n, m, _stream()))
+    return gated_state_scan(x, oq, ok, ov, *args, m, decay, oa, per_channel, first, seg_start, ids, nseg, **kw)
 
 
 def delta_rule_prep(c, G: int, n: int, q_scale: float, unit_eps: float, rows, oa: int, ob: int, a_log, dt_bias, H: int):

@@ -2,7 +2,9 @@
 
 Both keep, per head, a state ``S`` (``key_dim x value_dim``, float32 in both precisions, zero at a request's start) in the
 request's slot and advance it token by token with one kernel (``ops.gated_state_scan``), whose sums run in one order
-whatever the step's cut.
+whatever the step's cut.  A step that brings a portion of ``2 * SEGMENT`` tokens or more walks its portions in segments
+side by side (over a segment the state goes ``S -> M S + B``; ``ops.gated_state_scan_segments``); results then differ
+from the walk in one piece by float32 rounding.
 
 ``GatedDelta`` (the gated delta rule): with ``x`` the mixer's input,
 
@@ -30,6 +32,17 @@ import torch
 
 from .base import MATRIX, VECTOR, Part, SlotState, TensorSpec
 from .registry import register
+
+
+SEGMENT = 128      # tokens a segment: a step that brings a portion of twice as many walks its portions in segments
+
+
+def _scan(ops, ctx, args, state, **kw):
+    """The recurrence over this step's tokens: token by token a sequence, or, when a long portion is among them, the
+    portions' segments side by side."""
+    if not ctx.all_single and ctx.max_q_len >= 2 * SEGMENT:
+        return ops.gated_state_scan_segments(*args, state, ctx.q_lens, ctx.slots, SEGMENT, **kw)
+    return ops.gated_state_scan(*args, state, ctx.q_start, ctx.slots, ctx.nseq, **kw)
 
 
 def _stacked(ws, pad_to: int = 16):
@@ -97,8 +110,7 @@ class GatedDelta(Part):
             gates = ops.delta_rule_prep(qkv, G, n, float(n) ** -0.5, s.unit_eps, rows, C + H * m + H, C + H * m,
                                         self.a_log, self.dt_bias, H)
         with rt.stage("delta_state"):
-            o = ops.gated_state_scan(qkv, 0, G * n, 2 * G * n, H, G, n, m, gates, 0, False, cache.state["state"],
-                                     ctx.q_start, ctx.slots, ctx.nseq, beta=gates, ob=H)
+            o = _scan(ops, ctx, (qkv, 0, G * n, 2 * G * n, H, G, n, m, gates, 0, False), cache.state["state"], beta=gates, ob=H)
         with rt.stage("delta_norm"):
             y = ops.gated_outnorm(o, rows, C, self.norm_weight, s.eps, H, m, False, "silu", rt.dtype)
         return rt.linear(y, self.w_out, out_dtype=out_dtype)
@@ -152,8 +164,8 @@ class GatedLinear(Part):
             alpha = rt.linear(rt.linear(x, self.w_down), self.w_up, self.b_up, out_dtype=torch.float32)
             ops.channel_decay(alpha, s.tau)
         with rt.stage("decay_state"):
-            o = ops.gated_state_scan(rows, 0, H * n, 2 * H * n, H, H, n, m, alpha, 0, True, cache.state["state"],
-                                     ctx.q_start, ctx.slots, ctx.nseq, q_scale=float(n) ** -0.5)
+            o = _scan(ops, ctx, (rows, 0, H * n, 2 * H * n, H, H, n, m, alpha, 0, True), cache.state["state"],
+                      q_scale=float(n) ** -0.5)
         with rt.stage("decay_norm"):
             y = ops.gated_outnorm(o, rows, 2 * H * n + H * m, self.norm_weight, s.eps, H, m, False, "silu", rt.dtype)
         return rt.linear(y, self.w_out, out_dtype=out_dtype)

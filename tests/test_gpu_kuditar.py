@@ -279,7 +279,7 @@ def test_cache_write_with_a_plain_norm_a_partial_turn_wider_rows_and_blended_val
         assert float((pg.v[page, :, row].double().cpu() - v[t]).abs().max()) <= tol(dtype, v)
 
 
-def scan_case(ops, dtype, H, G, n, m, lens, cuts, per_channel, delta, seed=0, slow=False, meet=None):
+def scan_case(ops, dtype, H, G, n, m, lens, cuts, per_channel, delta, seed=0, slow=False, meet=None, segment=0):
     """The recurrence over sequences of ``lens`` tokens fed in the pieces ``cuts[s]``, states in shuffled slots.  Returns
     the kernel's rows and the plain recurrence's, per sequence, and the states left."""
     g = gen(seed)
@@ -311,9 +311,14 @@ def scan_case(ops, dtype, H, G, n, m, lens, cuts, per_channel, delta, seed=0, sl
         live = [s for s in range(len(lens)) if step < len(cuts[s])]
         sizes = [cuts[s][step] for s in live]
         cat = lambda parts: torch.cat([parts[s][done[s]:done[s] + k] for s, k in zip(live, sizes)]).to(DEV)
-        y = ops.gated_state_scan(cat(xs), junk, junk + G * n, junk + 2 * G * n, H, G, n, m, cat(decs), 3, per_channel, st,
-                                 i32(starts_of(sizes)), i32([slots[s] for s in live]), len(live), q_scale=0.5,
-                                 beta=cat(betas) if delta else None, ob=2)
+        if segment:       # the portions' segments side by side
+            y = ops.gated_state_scan_segments(cat(xs), junk, junk + G * n, junk + 2 * G * n, H, G, n, m, cat(decs), 3,
+                                              per_channel, st, sizes, i32([slots[s] for s in live]), segment, q_scale=0.5,
+                                              beta=cat(betas) if delta else None, ob=2)
+        else:
+            y = ops.gated_state_scan(cat(xs), junk, junk + G * n, junk + 2 * G * n, H, G, n, m, cat(decs), 3, per_channel, st,
+                                     i32(starts_of(sizes)), i32([slots[s] for s in live]), len(live), q_scale=0.5,
+                                     beta=cat(betas) if delta else None, ob=2)
         at = 0
         for s, k in zip(live, sizes):
             got[s].append(y[at:at + k].double().cpu())
@@ -363,10 +368,29 @@ def test_recurrences_over_unequal_sequences_and_any_cut(ops, dtype, H, G, n, m, 
         assert torch.equal(sa[slots_a[s]], sb[slots_b[s]])
 
 
-@pytest.mark.parametrize("cuts", [[[420]], [[330] + [1] * 90], [[7] * 60]])
-def test_a_state_keeps_what_it_was_given_hundreds_of_tokens_before(ops, cuts):
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,n,m,seg", [(4, 2, 16, 24, 32), (2, 2, 64, 64, 64), (2, 1, 128, 128, 128), (5, 5, 6, 14, 16), (3, 1, 40, 70, 50)])
+@pytest.mark.parametrize("per_channel,delta", [(False, True), (True, False)])
+def test_recurrences_in_segments_side_by_side(ops, dtype, H, G, n, m, seg, per_channel, delta):
+    """Portions of several segments beside short ones and single tokens; portions that start from states which earlier
+    steps left; the states left behind against the walk in one piece."""
+    if per_channel:
+        G = H
+    lens = [5 * seg + 3, 1, 2 * seg, seg + 9]
+    pieces = [[3 * seg + 1, 1, 2 * seg + 1], [1], [seg - 1, seg + 1], [seg + 9]]
+    whole = [[L] for L in lens]
+    a, want, sa, slots_a = scan_case(ops, dtype, H, G, n, m, lens, whole, per_channel, delta, seed=n + m)
+    b, _, sb, slots_b = scan_case(ops, dtype, H, G, n, m, lens, pieces, per_channel, delta, seed=n + m, segment=seg)
+    for s in range(len(lens)):
+        assert float((b[s] - want[s]).abs().max()) <= tol(torch.float32, want[s], 5e-5), s
+        assert float((sb[slots_b[s]] - sa[slots_a[s]]).abs().max()) <= tol(torch.float32, sa[slots_a[s]], 5e-5), s
+
+
+@pytest.mark.parametrize("cuts,seg", [([[420]], 0), ([[330] + [1] * 90], 0), ([[7] * 60], 0), ([[420]], 64), ([[290, 130]], 32)])
+def test_a_state_keeps_what_it_was_given_hundreds_of_tokens_before(ops, cuts, seg):
     for per_channel, delta in ((False, True), (True, False)):
-        got, want, _, _ = scan_case(ops, torch.float32, 2, 2, 8, 6, [420], cuts, per_channel, delta, seed=5, slow=True, meet=(20, 400))
+        got, want, _, _ = scan_case(ops, torch.float32, 2, 2, 8, 6, [420], cuts, per_channel, delta, seed=5, slow=True, meet=(20, 400),
+                                    segment=seg)
         assert float(want[0][400].abs().max()) > 10 * float(want[0][399].abs().max())      # the meeting shows
         assert float((got[0] - want[0]).abs().max()) <= tol(torch.float32, want[0], 3e-5)
 
@@ -572,6 +596,32 @@ def test_mixers_whole_token_by_token_in_portions_and_in_batches(dtype, kind, kw)
     assert float((out[0] - plain(y)[29]).abs().max()) <= bound
     assert float((out[1:21] - want[50:70]).abs().max()) <= bound
     assert float((out[21:] - plain(u)).abs().max()) <= bound
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind,kw", [("delta", dict()), ("delta", dict(W=128, H=2, G=2, n=64, m=64, taps=4)), ("decay", dict()),
+                                     ("decay", dict(W=128, H=2, n=128, m=128, r=16, tau=16.0)), ("pair", dict())])
+def test_recurrent_mixers_with_portions_long_enough_for_segments(dtype, kind, kw):
+    """A prompt of several segments whole; the same in two long portions and single tokens; a long portion of one request
+    beside a single token of another."""
+    h, plain = mixer_harness(kind, dtype, num_pages=128, **kw)
+    W = kw.get("W", 96)
+    T = 700
+    x = torch.randn(T, W, generator=gen(43)).to(dtype)
+    want = plain(x)
+    bound = tol(dtype, want, 5e-5, 3e-2)
+    assert float((h.mixer(x, [("whole", T)]) - want).abs().max()) <= bound
+    got = [h.mixer(x[:300], [("cut", 300)]), h.mixer(x[300:301], [("cut", 1)]), h.mixer(x[301:690], [("cut", 389)])]
+    got += [h.mixer(x[i:i + 1], [("cut", 1)]) for i in range(690, T)]
+    assert float((torch.cat(got) - want).abs().max()) <= bound
+    h.manager.release("whole")
+    h.manager.release("cut")
+    y = torch.randn(30, W, generator=gen(44)).to(dtype)
+    h.mixer(y[:29], [("b", 29)])
+    h.mixer(x[:130], [("a", 130)])
+    out = h.mixer(torch.cat([y[29:30], x[130:500]]), [("b", 1), ("a", 370)])
+    assert float((out[0] - plain(y)[29]).abs().max()) <= bound
+    assert float((out[1:] - want[130:500]).abs().max()) <= bound
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
